@@ -9,7 +9,7 @@
 
 namespace mxs {
 void launch_resid_update(float*, const void*, long, const void*, const void*, long, const void*, const void*, int,
-                         const void*, void*, int, int, float, bool, hipStream_t);
+                         const void*, void*, int, int, float, float, float, bool, hipStream_t);
 void launch_cast_into(void*, long, const float*, int, int, bool, hipStream_t);
 void launch_relu_sq(void*, const void*, long, bool, hipStream_t);
 void launch_softcap(float*, const void*, long, int, int, float, bool, hipStream_t);
@@ -18,7 +18,8 @@ void launch_gate_linear(float*, const void*, long, const void*, const void*, int
 void launch_kv_write(void*, long, const void*, long, const void*, long, const int64_t*, int, int, int, int, int, int,
                      int, bool, hipStream_t);
 bool launch_window_attention(void*, const void*, long, const void*, long, const int*, int, const int*, const int*, int,
-                             int, int, int, int, int, int, int, int, float, int, int, int, const float*, bool, hipStream_t);
+                             int, int, int, int, int, int, int, int, float, int, int, int, const float*, int, bool,
+                             hipStream_t);
 bool launch_matrix_scan(float*, const void*, long, const void*, long, const void*, long, const float*, const float*,
                         float*, long, const int*, long, const int*, const int*, int, int, int, int, int, int, float,
                         float, bool, bool, int, int, float*, float*, long, hipStream_t);
@@ -34,6 +35,16 @@ void launch_causal_conv(void*, const void*, long, const void*, const void*, floa
 void launch_gated_norm(void*, long, const float*, const void*, long, const void*, int, int, int, int, float, int, int,
                        float, bool, hipStream_t);
 bool launch_column_scan(const ScanArgs&, int, bool, bool, hipStream_t);
+void launch_latent_prep(void*, const void*, long, const void*, long, const int64_t*, const int64_t*, void*, long, int, int,
+                        int, int, int, int, const float*, const void*, const void*, float, bool, hipStream_t);
+void launch_rope_half_into(void*, long, const void*, long, const int64_t*, int, int, int, int, int, int, const float*, int,
+                           bool, hipStream_t);
+void launch_route_topk(float*, int*, const float*, int, int, int, bool, hipStream_t);
+void launch_capped_glu(void*, const void*, long, int, int, float, float, bool, hipStream_t);
+bool launch_expert_align(int*, int*, const int*, int, int, hipStream_t);
+void launch_gather_scaled(void*, const void*, long, const float*, const int*, int, int, int, bool, hipStream_t);
+void launch_spread_scaled(void*, const void*, long, const float*, const int*, int, int, int, int, bool, hipStream_t);
+void launch_expert_combine(void*, const void*, const int*, int, int, long, const void*, long, int, bool, hipStream_t);
 }  // namespace mxs
 
 namespace {
@@ -74,7 +85,7 @@ float* f32(const at::Tensor& t, const char* name) {
 }
 
 void resid_update(at::Tensor x, OptT a, OptT wa, OptT b, OptT wb, OptT bias, bool assign, OptT norm_w, OptT h,
-                  double eps) {
+                  double eps, double a_scale, double w_offset) {
   float* xp = f32(x, "x");
   TORCH_CHECK(x.dim() == 2, "x: [T, W]");
   const int64_t T = x.size(0), W = x.size(1);
@@ -95,7 +106,8 @@ void resid_update(at::Tensor x, OptT a, OptT wa, OptT b, OptT wb, OptT bias, boo
   mxs::launch_resid_update(xp, ap, a.has_value() ? a->stride(0) : 0, vec(wa, bf, W, "wa"), bp,
                            b.has_value() ? b->stride(0) : 0, vec(wb, bf, W, "wb"), vec(bias, bf, W, "bias"), assign,
                            vec(norm_w, bf, W, "norm_w"), hp, static_cast<int>(T), static_cast<int>(W),
-                           static_cast<float>(eps), bf, stream());
+                           static_cast<float>(eps), static_cast<float>(a_scale), static_cast<float>(w_offset), bf,
+                           stream());
 }
 
 void cast_into(at::Tensor dst, at::Tensor x) {
@@ -167,7 +179,8 @@ void kv_write(at::Tensor cache, at::Tensor k, at::Tensor v, at::Tensor slots, in
 
 void window_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor block_tables, at::Tensor qsl,
                       at::Tensor seq_lens, int64_t koff, int64_t voff, int64_t H, int64_t G, int64_t dk, int64_t dv,
-                      int64_t bs, double scale, int64_t window, int64_t keep, int64_t max_query_len, OptT sink) {
+                      int64_t bs, double scale, int64_t window, int64_t keep, int64_t max_query_len, OptT sink,
+                      int64_t v_stride) {
   const bool bf = is_bf(q);
   const float* sinkp = nullptr;
   if (sink.has_value()) {
@@ -175,7 +188,13 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor
     TORCH_CHECK(sink->numel() == H, "sink: fp32 [H]");
   }
   const int64_t T = q.size(0), S = seq_lens.numel();
-  check_cache(cache, bf, koff, voff, G, dk, dv, bs);
+  if (v_stride > 0 && v_stride != dv) {  // values are a slice of a wider cached row of the one kv head
+    TORCH_CHECK(G == 1 && v_stride >= dv, "strided value rows: one kv head, stride >= dv");
+    check_cache(cache, bf, koff, voff, G, dk, 0, bs);
+    TORCH_CHECK(voff >= 0 && voff + (bs - 1) * v_stride + dv <= cache.size(1), "value rows reach past the cache block");
+  } else {
+    check_cache(cache, bf, koff, voff, G, dk, dv, bs);
+  }
   TORCH_CHECK(G >= 1 && H % G == 0, "query heads must divide over kv heads");
   TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv &&
               is_bf(out) == bf, "out: [T, H*dv]");
@@ -187,7 +206,7 @@ void window_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor
       i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(koff),
       static_cast<int>(voff), static_cast<int>(H), static_cast<int>(G), static_cast<int>(dk), static_cast<int>(dv),
       static_cast<int>(bs), static_cast<float>(scale), static_cast<int>(window), static_cast<int>(keep),
-      static_cast<int>(std::min<int64_t>(max_query_len, T)), sinkp, bf, stream());
+      static_cast<int>(std::min<int64_t>(max_query_len, T)), sinkp, static_cast<int>(v_stride), bf, stream());
   TORCH_CHECK(ok, "window_attention: head sizes beyond what the kernel holds (dv <= 512)");
 }
 
@@ -413,6 +432,113 @@ void delta_scan(at::Tensor out, at::Tensor q, at::Tensor k, at::Tensor v, at::Te
               q_scale, unit_eps, piece, npieces, sc_local, sc_start, OptT(), mode, max_q);
 }
 
+// ---- latent attention, routed experts (latent_experts.hip)
+const int64_t* i64c(const at::Tensor& t, int64_t n, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kLong && t.is_contiguous() && t.numel() == n, name,
+              ": expected ", n, " contiguous int64");
+  return t.data_ptr<int64_t>();
+}
+
+void latent_prep(at::Tensor cq, at::Tensor dq, at::Tensor dkv, at::Tensor positions, at::Tensor slots, at::Tensor cache,
+                 int64_t koff, int64_t rank, int64_t bs, at::Tensor freqs, at::Tensor q_norm, at::Tensor kv_norm,
+                 double eps) {
+  const bool bf = is_bf(dq);
+  const int64_t T = dq.size(0), qr = dq.size(1), nf = freqs.numel(), dk = rank + 2 * nf;
+  TORCH_CHECK(rank >= 1 && bs >= 1, "rank and block size must be positive");
+  check_cache(cache, bf, koff, koff, 1, dk, 0, bs);
+  TORCH_CHECK(cq.is_cuda() && cq.is_contiguous() && cq.dim() == 2 && cq.size(0) == T && cq.size(1) == qr && is_bf(cq) == bf,
+              "cq: contiguous [T, q_rank]");
+  mxs::launch_latent_prep(cq.data_ptr(), mat(dq, bf, T, qr, "dq"), dq.stride(0), mat(dkv, bf, T, dk, "dkv"), dkv.stride(0),
+                          i64c(positions, T, "positions"), i64c(slots, T, "slot_mapping"), cache.data_ptr(), cache.stride(0),
+                          static_cast<int>(T), static_cast<int>(koff), static_cast<int>(qr), static_cast<int>(rank),
+                          static_cast<int>(nf), static_cast<int>(bs), f32(freqs, "freqs"),
+                          vec(OptT(q_norm), bf, qr, "q_norm"), vec(OptT(kv_norm), bf, rank, "kv_norm"),
+                          static_cast<float>(eps), bf, stream());
+}
+
+void rope_half_into(at::Tensor out, at::Tensor x, at::Tensor positions, int64_t heads, int64_t x_dim, int64_t x_col,
+                    int64_t out_dim, int64_t out_col, at::Tensor freqs) {
+  const bool bf = is_bf(x);
+  const int64_t T = x.size(0), nf = freqs.numel();
+  TORCH_CHECK(x_col >= 0 && out_col >= 0 && x_col + 2 * nf <= x_dim && out_col + 2 * nf <= out_dim,
+              "the rotated columns lie outside a head");
+  mxs::launch_rope_half_into(const_cast<void*>(mat(out, bf, T, heads * out_dim, "out")), out.stride(0),
+                             mat(x, bf, T, heads * x_dim, "x"), x.stride(0), i64c(positions, T, "positions"),
+                             static_cast<int>(T), static_cast<int>(heads), static_cast<int>(x_dim), static_cast<int>(x_col),
+                             static_cast<int>(out_dim), static_cast<int>(out_col), f32(freqs, "freqs"), static_cast<int>(nf),
+                             bf, stream());
+}
+
+void route_topk(at::Tensor w, at::Tensor ids, at::Tensor logits, bool renorm) {
+  const float* lp = f32(logits, "logits");
+  TORCH_CHECK(logits.dim() == 2 && w.dim() == 2 && ids.dim() == 2, "logits [T, E], w / ids [T, k]");
+  const int64_t T = logits.size(0), E = logits.size(1), k = w.size(1);
+  TORCH_CHECK(k >= 1 && k <= E && w.size(0) == T && ids.size(0) == T && ids.size(1) == k, "1 <= k <= E; w, ids [T, k]");
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kInt && ids.is_contiguous(), "ids: contiguous int32");
+  mxs::launch_route_topk(f32(w, "w"), ids.data_ptr<int>(), lp, static_cast<int>(T), static_cast<int>(E),
+                         static_cast<int>(k), renorm, stream());
+}
+
+void capped_glu(at::Tensor out, at::Tensor gu, double limit, double alpha) {
+  const bool bf = is_bf(gu);
+  TORCH_CHECK(gu.is_cuda() && gu.dim() == 2 && gu.size(1) % 2 == 0 && (gu.size(1) == 1 || gu.stride(1) == 1), "gu: [R, 2F]");
+  const int64_t R = gu.size(0), F = gu.size(1) / 2;
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == R && out.size(1) == F &&
+              is_bf(out) == bf, "out: contiguous [R, F]");
+  mxs::launch_capped_glu(out.data_ptr(), gu.data_ptr(), gu.stride(0), static_cast<int>(R), static_cast<int>(F),
+                         static_cast<float>(limit), static_cast<float>(alpha), bf, stream());
+}
+
+void expert_align(at::Tensor offs, at::Tensor inv, at::Tensor ids, int64_t E) {
+  const int64_t n = ids.numel();
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kInt && ids.is_contiguous(), "ids: contiguous int32");
+  TORCH_CHECK(E >= 1 && n < (1LL << 30), "expert count / pair count out of range");
+  int* op = const_cast<int*>(i32(offs, E + 1, "offs"));
+  int* ip = const_cast<int*>(i32(inv, n, "inv"));
+  TORCH_CHECK(mxs::launch_expert_align(op, ip, ids.data_ptr<int>(), static_cast<int>(n), static_cast<int>(E), stream()),
+              "expert_align: more experts than the kernel's counters hold");
+}
+
+void gather_scaled(at::Tensor xs, at::Tensor h, at::Tensor w, at::Tensor inv) {
+  const bool bf = is_bf(h);
+  TORCH_CHECK(w.dim() == 2 && h.dim() == 2 && w.size(0) == h.size(0), "h [T, W], w [T, k]");
+  const int64_t T = h.size(0), W = h.size(1), k = w.size(1);
+  TORCH_CHECK(xs.is_cuda() && xs.is_contiguous() && xs.dim() == 2 && xs.size(0) == T * k && xs.size(1) == W &&
+              is_bf(xs) == bf, "xs: contiguous [T*k, W]");
+  // inv comes from expert_align over the same pairs: a permutation of 0 .. T*k-1
+  mxs::launch_gather_scaled(xs.data_ptr(), mat(h, bf, T, W, "h"), h.stride(0), f32(w, "w"), i32(inv, T * k, "inv"),
+                            static_cast<int>(T * k), static_cast<int>(k), static_cast<int>(W), bf, stream());
+}
+
+void spread_scaled(at::Tensor xs, at::Tensor h, at::Tensor w, at::Tensor ids) {
+  const bool bf = is_bf(h);
+  TORCH_CHECK(w.dim() == 2 && h.dim() == 2 && w.size(0) == h.size(0) && xs.dim() == 3, "h [T, W], w [T, k], xs [E, T, W]");
+  const int64_t T = h.size(0), W = h.size(1), k = w.size(1), E = xs.size(0);
+  TORCH_CHECK(xs.is_cuda() && xs.is_contiguous() && xs.size(1) == T && xs.size(2) == W && is_bf(xs) == bf,
+              "xs: contiguous [E, T, W]");
+  TORCH_CHECK(E <= 65535, "more experts than a grid dimension holds");
+  mxs::launch_spread_scaled(xs.data_ptr(), mat(h, bf, T, W, "h"), h.stride(0), f32(w, "w"), i32(ids, T * k, "ids"),
+                            static_cast<int>(T), static_cast<int>(E), static_cast<int>(k), static_cast<int>(W), bf,
+                            stream());
+}
+
+void expert_combine(at::Tensor out, at::Tensor ys, OptT index, int64_t k, OptT extra, int64_t row_stride) {
+  const bool bf = is_bf(ys);
+  TORCH_CHECK(ys.is_cuda() && ys.is_contiguous() && ys.dim() == 2 && out.is_cuda() && out.is_contiguous() &&
+              out.dim() == 2 && out.size(1) == ys.size(1) && is_bf(out) == bf, "ys [R, W], out [T, W]");
+  const int64_t T = out.size(0), W = out.size(1), R = ys.size(0);
+  const int* ip = nullptr;
+  if (index.has_value()) {
+    ip = i32(*index, T * k, "index");  // entries are rows of ys: expert_align's places, < T*k <= R
+    TORCH_CHECK(T * k <= R, "index reaches past ys");
+  } else {
+    TORCH_CHECK(k >= 1 && row_stride >= T && (k - 1) * row_stride + T <= R, "the k slabs reach past ys");
+  }
+  const void* ep = extra.has_value() ? mat(*extra, bf, T, W, "extra") : nullptr;
+  mxs::launch_expert_combine(out.data_ptr(), ys.data_ptr(), ip, static_cast<int>(T), static_cast<int>(k), row_stride, ep,
+                             extra.has_value() ? extra->stride(0) : 0, static_cast<int>(W), bf, stream());
+}
+
 }  // namespace
 
 PYBIND11_MODULE(_M, m) {
@@ -434,4 +560,12 @@ PYBIND11_MODULE(_M, m) {
   m.def("gated_norm", &gated_norm);
   m.def("ssd_scan", &ssd_scan);
   m.def("delta_scan", &delta_scan);
+  m.def("latent_prep", &latent_prep);
+  m.def("rope_half_into", &rope_half_into);
+  m.def("route_topk", &route_topk);
+  m.def("capped_glu", &capped_glu);
+  m.def("expert_align", &expert_align);
+  m.def("gather_scaled", &gather_scaled);
+  m.def("spread_scaled", &spread_scaled);
+  m.def("expert_combine", &expert_combine);
 }

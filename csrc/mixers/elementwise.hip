@@ -13,7 +13,7 @@ __global__ void __launch_bounds__(256) resid_update_kernel(float* __restrict__ x
                                                            long b_stride, const T* __restrict__ wb,
                                                            const T* __restrict__ bias, int assign,
                                                            const T* __restrict__ norm_w, T* __restrict__ h, int W,
-                                                           float eps) {
+                                                           float eps, float a_scale, float w_offset) {
   __shared__ float scratch[16];
   const long row = blockIdx.x;
   float* xr = x + row * W;
@@ -34,7 +34,7 @@ __global__ void __launch_bounds__(256) resid_update_kernel(float* __restrict__ x
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float xv = xr[c];
     if (ar) {
-      float d = ldf(ar + c);
+      float d = ldf(ar + c) * a_scale;
       if (wa) d = d * ra * ldf(wa + c);
       if (br) d = 0.5f * (d + ldf(br + c) * rb * ldf(wb + c));
       if (bias) d += ldf(bias + c);
@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(256) resid_update_kernel(float* __restrict__ x
   if (norm_w == nullptr) return;
   const float inv = rsqrtf(block_sum(ss, scratch) / static_cast<float>(W) + eps);
   T* hr = h + row * W;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) stf(hr + c, xr[c] * inv * ldf(norm_w + c));  // own writes
+  for (int c = threadIdx.x; c < W; c += blockDim.x) stf(hr + c, xr[c] * inv * (w_offset + ldf(norm_w + c)));  // own writes
 }
 
 template <typename T>
@@ -151,11 +151,11 @@ __global__ void __launch_bounds__(256) kv_write_kernel(T* __restrict__ cache, lo
 
 void launch_resid_update(float* x, const void* a, long a_stride, const void* wa, const void* b, long b_stride,
                          const void* wb, const void* bias, int assign, const void* norm_w, void* h, int rows, int W,
-                         float eps, bool bf, hipStream_t st) {
+                         float eps, float a_scale, float w_offset, bool bf, hipStream_t st) {
   if (rows == 0) return;
   MIX_DISPATCH(bf, hipLaunchKernelGGL(resid_update_kernel<T>, dim3(rows), dim3(256), 0, st, x, (const T*)a, a_stride,
                                       (const T*)wa, (const T*)b, b_stride, (const T*)wb, (const T*)bias, assign,
-                                      (const T*)norm_w, (T*)h, W, eps));
+                                      (const T*)norm_w, (T*)h, W, eps, a_scale, w_offset));
   MXS_CHECK_LAUNCH();
 }
 

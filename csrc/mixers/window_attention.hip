@@ -19,7 +19,7 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long block_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep, bool vec,
-    const float* __restrict__ sink) {
+    const float* __restrict__ sink, int vs) {
   extern __shared__ float lds[];
   float* qs = lds;                      // [dk]
   float* p = qs + ((dk + 3) & ~3);      // [kKeyTile]
@@ -64,7 +64,7 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
     for (int n = wid; n < nt; n += 4) {
       const int nn = t0 + n;
       const int j = nn < nA ? nn : lo + (nn - nA);
-      const T* vp = cache + static_cast<long>(bt[j / bs]) * block_stride + voff + (static_cast<long>(g) * bs + j % bs) * dv;
+      const T* vp = cache + static_cast<long>(bt[j / bs]) * block_stride + voff + (static_cast<long>(g) * bs + j % bs) * vs;
       const float pn = p[n];
 #pragma unroll
       for (int c = 0; c < kMaxVChunks; ++c) {
@@ -114,7 +114,7 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
     T* __restrict__ out, const T* __restrict__ q, long q_stride, const T* __restrict__ cache, long block_stride,
     const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     int S, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep, int nsplit,
-    const float* __restrict__ sink) {
+    const float* __restrict__ sink, int vs) {
   constexpr int EL = El<T>::N;
   extern __shared__ float lds[];
   float* p = lds;                      // [RM][kKeyTile]
@@ -216,7 +216,7 @@ __global__ void __launch_bounds__(256) window_attention_rows_kernel(
     for (int n = slot; n < nt; n += 32) {
       const int nn = t0 + n;
       const int j = nn < nA ? nn : lo + (nn - nA);
-      const T* vp = cache + static_cast<long>(bt[j / bs]) * block_stride + voff + (static_cast<long>(g) * bs + j % bs) * dv;
+      const T* vp = cache + static_cast<long>(bt[j / bs]) * block_stride + voff + (static_cast<long>(g) * bs + j % bs) * vs;
       float pn[RM];
 #pragma unroll
       for (int r = 0; r < RM; ++r) pn[r] = p[r * kKeyTile + n];
@@ -416,11 +416,12 @@ __global__ void __launch_bounds__(256) window_attention_mfma_kernel(
 bool launch_window_attention(void* out, const void* q, long q_stride, const void* cache, long block_stride,
                              const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S,
                              int rows, int koff, int voff, int H, int G, int dk, int dv, int bs, float scale,
-                             int window, int keep, int max_q, const float* sink, bool bf, hipStream_t st) {
+                             int window, int keep, int max_q, const float* sink, int vs, bool bf, hipStream_t st) {
   if (rows == 0 || S == 0) return true;
+  if (vs <= 0) vs = dv;  // value rows back to back
   // prompt chunks in bf16 with MFMA-shaped heads: the matrix-core form (rows of a mixed step's single
   // tokens ride along as 1-row tiles); everything else the scalar form below
-  if (bf && max_q >= 16 && bs == 16 && dk % 16 == 0 && dv % 16 == 0 && dk <= 128 && dv <= 128 && q_stride % 4 == 0 &&
+  if (bf && vs == dv && max_q >= 16 && bs == 16 && dk % 16 == 0 && dv % 16 == 0 && dk <= 128 && dv <= 128 && q_stride % 4 == 0 &&
       reinterpret_cast<uintptr_t>(q) % 8 == 0 && koff % 8 == 0 && voff % 8 == 0 && block_stride % 8 == 0) {
     const dim3 grid((max_q + 63) / 64, H, S);
 #define MIX_WA(KSM, VTM)                                                                                              \
@@ -438,7 +439,7 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
   const bool vec = dk % el == 0 && koff % el == 0 && block_stride % el == 0;
   const size_t shm = (((dk + 3) & ~3) + kKeyTile + 4 * dv) * sizeof(float);
   if (shm > 60 * 1024) return false;
-  if (vec && dv % el == 0 && voff % el == 0 && dk <= 256 && dv <= 256) {  // rows of whole 16-byte pieces
+  if (vec && dv % el == 0 && voff % el == 0 && vs % el == 0 && dk <= 256 && dv <= 256) {  // rows of whole 16-byte pieces
     const int stretch = 8 * el, need = (std::max(dk, dv) + stretch - 1) / stretch;  // 128-byte stretches of a row
     const int R = H / G;
 #define MIX_ROWS(TT, NC, RM)                                                                                          \
@@ -447,7 +448,7 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
     const size_t sh = (static_cast<size_t>(RM) * kKeyTile + 4 * RM * dv) * sizeof(float);                             \
     hipLaunchKernelGGL((window_attention_rows_kernel<TT, NC, RM>), dim3(rows, G * nsplit), dim3(256), sh, st, (TT*)out, \
                        (const TT*)q, q_stride, (const TT*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, \
-                       S, koff, voff, H, G, dk, dv, bs, scale, window, keep, nsplit, sink);                            \
+                       S, koff, voff, H, G, dk, dv, bs, scale, window, keep, nsplit, sink, vs);                        \
   } while (0)
 #define MIX_ROWS_T(TT)                                          \
   do {                                                          \
@@ -466,11 +467,11 @@ bool launch_window_attention(void* out, const void* q, long q_stride, const void
   if (bf)
     hipLaunchKernelGGL(window_attention_kernel<bf16_t>, dim3(rows, H), dim3(256), shm, st, (bf16_t*)out, (const bf16_t*)q,
                        q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, koff,
-                       voff, H, G, dk, dv, bs, scale, window, keep, vec, sink);
+                       voff, H, G, dk, dv, bs, scale, window, keep, vec, sink, vs);
   else
     hipLaunchKernelGGL(window_attention_kernel<float>, dim3(rows, H), dim3(256), shm, st, (float*)out, (const float*)q,
                        q_stride, (const float*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, koff,
-                       voff, H, G, dk, dv, bs, scale, window, keep, vec, sink);
+                       voff, H, G, dk, dv, bs, scale, window, keep, vec, sink, vs);
   MXS_CHECK_LAUNCH();
   return true;
 }

@@ -18,7 +18,7 @@ from typing import Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str  # "llama" | "qwen3" | "mixtral" | "voletar" | "tapasun"
+    arch: str  # "llama" | "qwen3" | "mixtral" | "voletar" | "tapasun" | "momuvik"
     hidden_size: int
     intermediate_size: int
     num_layers: int
@@ -40,7 +40,7 @@ class ModelConfig:
     bos_token_id: Optional[int] = None
     eos_token_ids: list = field(default_factory=list)
     chat_template: str = "llama3"
-    # designs whose layers differ from one another (arch "voletar", "tapasun"): the checkpoint's own
+    # designs whose config lists their layers (arch "voletar", "tapasun", "momuvik"): the checkpoint's own
     # config.json structure -- per-layer mixer type and sizes, norm eps and the design's other
     # constants -- as the design's module (mxserve/models/<arch>.py) reads it.  None for the uniform
     # transformer families.
@@ -246,7 +246,50 @@ _reg(tapasun_config("tiny-tapasun", {
                            "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 64}}}}]}))
 
 
+def momuvik_config(name: str, d: dict) -> ModelConfig:
+    """A Momuvik checkpoint's config.json: `width`, `vocab`, `embedding.scale`, `norm.eps`, `residual_mult`,
+    `layers` (each with `type` latent_attention, `mixer`, `mlp` dense | moe | null, optionally `weights_of`).
+    The uniform fields are filled from the first layer for the code that sizes things from them."""
+    layers = d["layers"]
+    att = layers[0]["mixer"]
+    ffs = [int(l["mlp"]["ff"]) if l["mlp"].get("kind", "dense") == "dense" else int(l["mlp"]["expert"]["ff"])
+           for l in layers if l.get("mlp")]
+    moes = [l["mlp"]["router"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "moe"]
+    keep = {k: d[k] for k in ("layers", "norm", "embedding", "residual_mult", "width", "vocab") if k in d}
+    return ModelConfig(
+        name=name, arch="momuvik", hidden_size=int(d["width"]), intermediate_size=max(ffs) if ffs else 0,
+        num_layers=len(layers), num_heads=int(att["heads"]), num_kv_heads=1,
+        head_dim=int(att["dim"]) + int(att["rot_dim"]), vocab_size=int(d["vocab"]),
+        rms_norm_eps=float((d.get("norm") or {}).get("eps", 1e-5)), tie_word_embeddings=True,
+        max_position_embeddings=int(d.get("max_position_embeddings", 1 << 20)),
+        num_experts=max((int(r["experts"]) for r in moes), default=0),
+        num_experts_per_tok=max((int(r["top"]) for r in moes), default=0),
+        bos_token_id=d.get("bos_token_id"), eos_token_ids=list(d.get("eos_token_ids") or []),
+        chat_template="chatml", arch_config=keep)
+
+
+def _latent(heads, dim, rot_dim, vdim, kv_rank, q_rank, scale, base=10000.0):
+    return {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+            "scale": scale, "rot": {"dims": rot_dim, "base": base}}
+
+
+# A small Momuvik (random weights): a dense and a routed feed-forward, a layer without one, shared weights.
+_reg(momuvik_config("tiny-momuvik", {
+    "architecture": "Momuvik", "width": 96, "vocab": 384, "norm": {"eps": 1e-5}, "embedding": {"scale": 6.0},
+    "residual_mult": 0.8,
+    "layers": [
+        {"type": "latent_attention", "mixer": _latent(4, 16, 8, 24, 32, 40, 0.2), "mlp": {"kind": "dense", "ff": 160}},
+        {"type": "latent_attention", "mixer": _latent(3, 24, 16, 16, 48, 24, 0.16, 5000.0),
+         "mlp": {"kind": "moe", "router": {"experts": 6, "top": 2}, "expert": {"ff": 48, "limit": 2.0},
+                 "shared": {"ff": 64, "limit": 1.2}}},
+        {"type": "latent_attention", "mixer": _latent(4, 16, 8, 24, 32, 40, 0.2), "mlp": {"kind": "dense", "ff": 160},
+         "weights_of": 0},
+        {"type": "latent_attention", "mixer": _latent(2, 32, 8, 32, 24, 32, 0.15), "mlp": None}]}))
+
+
 def _from_hf_json(name: str, d: dict) -> ModelConfig:
+    if d.get("architecture") == "Momuvik":
+        return momuvik_config(name, d)
     if d.get("architecture") == "Voletar":
         return voletar_config(name, d)
     if d.get("architecture") == "Tapasun":

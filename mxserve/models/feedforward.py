@@ -1,0 +1,135 @@
+"""Feed-forward sublayers that a layer-list design can be built from, each with its sizes and
+constants as parameters.  Like the mixers (mxserve/models/mixers.py) they name their checkpoint
+tensors, re-pack them once when the weights are loaded, and compute from a step's flattened batch.
+
+  GatedFF        W_down(act(W_gate h) * W_up h), gate and up as one projection; act = silu
+  CappedExpert   one small gated unit with clipped pre-activations: g = min(W_gate x, limit),
+                 u = clamp(W_up x, -limit, limit), W_down(g * sigmoid(alpha g) * (u + 1))
+  RoutedExperts  a sigmoid router (fp32) picks `top` of `experts` CappedExperts per token; the chosen
+                 scores weigh each expert's INPUT (optionally renormalised); an optional shared
+                 CappedExpert with its own size and limit sees every token unweighted
+
+The kernels are in mxserve/ops/seqmix.py (csrc/mixers/experts.hip on the GPU); the matrix products go
+through ops.linear and torch.bmm (hipBLASLt).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import ops
+from ..ops import seqmix
+
+
+class FeedForward:
+    def shapes(self) -> dict:
+        """Checkpoint tensor names -> shapes."""
+        raise NotImplementedError
+
+    def finish_weights(self, w: dict) -> None:
+        pass
+
+    def forward(self, h: torch.Tensor, w: dict) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class GatedFF(FeedForward):
+    def __init__(self, prefix: str, width: int, ff: int):
+        self.p, self.width, self.ff = prefix, width, int(ff)
+
+    def shapes(self) -> dict:
+        p = self.p
+        return {p + "gate": (self.ff, self.width), p + "up": (self.ff, self.width), p + "down": (self.width, self.ff)}
+
+    def finish_weights(self, w: dict) -> None:
+        p = self.p
+        w[p + "_gu"] = torch.cat([w.pop(p + "gate"), w.pop(p + "up")]).contiguous()
+
+    def forward(self, h: torch.Tensor, w: dict) -> torch.Tensor:
+        p = self.p
+        return ops.linear(seqmix.silu_mul(ops.linear(h, w[p + "_gu"])), w[p + "down"])
+
+
+class CappedExpert(FeedForward):
+    def __init__(self, prefix: str, width: int, ff: int, limit: float, alpha: float = 1.702):
+        self.p, self.width, self.ff = prefix, width, int(ff)
+        self.limit, self.alpha = float(limit), float(alpha)
+
+    def shapes(self) -> dict:
+        p = self.p
+        return {p + "gate": (self.ff, self.width), p + "up": (self.ff, self.width), p + "down": (self.width, self.ff)}
+
+    def finish_weights(self, w: dict) -> None:
+        p = self.p
+        w[p + "_gu"] = torch.cat([w.pop(p + "gate"), w.pop(p + "up")]).contiguous()
+
+    def forward(self, h: torch.Tensor, w: dict) -> torch.Tensor:
+        p = self.p
+        return ops.linear(seqmix.capped_glu(ops.linear(h, w[p + "_gu"]), self.limit, self.alpha), w[p + "down"])
+
+
+class RoutedExperts(FeedForward):
+    """Tensors: `<p>router` [E, width], `<p>e<i>.{gate,up,down}`, optionally `<p>shared.{gate,up,down}`.
+    Loaded as `<p>_gu` [E, 2 ff, width] and `<p>_down` [E, width, ff].
+
+    Two ways through the experts, both exact (a token never meets an expert it did not choose with
+    anything but a zero row, and a zero row gives a zero output: g = 0):
+      batched   every expert over all T rows of `spread_scaled` in two batched products -- no sorting
+                and no host round trip, so a captured single-token step can replay it; E / top times
+                the needed products, which steps of a few tokens do not feel (they stream the
+                experts' weights either way)
+      sorted    rows sorted by expert (expert_align, gather_scaled), one product pair per expert that
+                got rows (one host read of the E + 1 offsets), expert_combine gathers each token's rows
+    """
+
+    BATCHED_MAX_TOKENS = 32
+
+    def __init__(self, prefix: str, width: int, experts: int, top: int, ff: int, limit: float,
+                 shared: Optional[CappedExpert] = None, alpha: float = 1.702, renorm: bool = False):
+        if not 1 <= top <= experts:
+            raise ValueError(f"{prefix}: top {top} of {experts} experts")
+        self.p, self.width, self.E, self.top, self.ff = prefix, width, int(experts), int(top), int(ff)
+        self.limit, self.alpha, self.renorm, self.shared = float(limit), float(alpha), bool(renorm), shared
+
+    def shapes(self) -> dict:
+        p, sh = self.p, {self.p + "router": (self.E, self.width)}
+        for e in range(self.E):
+            sh[f"{p}e{e}.gate"] = sh[f"{p}e{e}.up"] = (self.ff, self.width)
+            sh[f"{p}e{e}.down"] = (self.width, self.ff)
+        if self.shared is not None:
+            sh.update(self.shared.shapes())
+        return sh
+
+    def finish_weights(self, w: dict) -> None:
+        p = self.p
+        w[p + "_gu"] = torch.stack([torch.cat([w.pop(f"{p}e{e}.gate"), w.pop(f"{p}e{e}.up")]) for e in range(self.E)]).contiguous()
+        w[p + "_down"] = torch.stack([w.pop(f"{p}e{e}.down") for e in range(self.E)]).contiguous()
+        if self.shared is not None:
+            self.shared.finish_weights(w)
+
+    def route(self, h: torch.Tensor, w: dict) -> tuple:
+        logits = seqmix.gate_linear(h, w[self.p + "router"], None)  # fp32 products and sums
+        return seqmix.route_topk(logits, self.top, self.renorm)
+
+    def forward(self, h: torch.Tensor, w: dict) -> torch.Tensor:
+        p, T = self.p, h.shape[0]
+        tw, ids = self.route(h, w)
+        extra = self.shared.forward(h, w) if self.shared is not None else None
+        gu, down = w[p + "_gu"], w[p + "_down"]
+        capturing = h.is_cuda and torch.cuda.is_current_stream_capturing()
+        if T <= self.BATCHED_MAX_TOKENS or capturing:
+            xs = seqmix.spread_scaled(h, tw, ids, self.E)  # [E, T, W]
+            a = seqmix.capped_glu(torch.bmm(xs, gu.transpose(1, 2)).view(self.E * T, -1), self.limit, self.alpha)
+            ys = torch.bmm(a.view(self.E, T, -1), down.transpose(1, 2))  # [E, T, W]
+            return seqmix.expert_combine(ys, None, self.E, T, extra, row_stride=T)
+        offs, inv = seqmix.expert_align(ids, self.E)
+        xs = seqmix.gather_scaled(h, tw, inv)
+        ys = torch.empty_like(xs)
+        o = offs.tolist()  # the one host read of this path
+        for e in range(self.E):
+            a0, a1 = o[e], o[e + 1]
+            if a1 > a0:
+                act = seqmix.capped_glu(ops.linear(xs[a0:a1], gu[e]), self.limit, self.alpha)
+                ys[a0:a1] = ops.linear(act, down[e])
+        return seqmix.expert_combine(ys, inv, self.top, T, extra)

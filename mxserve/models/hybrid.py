@@ -1,5 +1,5 @@
-"""What the designs whose layers differ from one another share (mxserve/models/voletar.py,
-mxserve/models/tapasun.py): the plan of layer runs with every run's place inside a cache block and a
+"""What the designs whose config lists their layers share (mxserve/models/voletar.py,
+mxserve/models/tapasun.py, mxserve/models/momuvik.py): the plan of layer runs with every run's place inside a cache block and a
 state slot, and the model surface the runner expects (weights in a flat dict, the mixers' input
 projections fused into one GEMM per layer, cache geometry from the plan).
 
@@ -18,7 +18,7 @@ from ..parallel.comm import get_tp
 from .config import ModelConfig
 from .mixers import Mixer
 
-HYBRID_ARCHS = ("voletar", "tapasun")
+HYBRID_ARCHS = ("voletar", "tapasun", "momuvik")
 
 
 def design_module(arch: str):
@@ -94,7 +94,7 @@ class HybridLM:
         if cfg.arch_config is None:
             raise ValueError(f"{name} needs the checkpoint's layer list (ModelConfig.arch_config)")
         if get_tp().tp_size != 1:
-            raise ValueError(f"{name} runs on one GPU per replica (its recurrent state is not sharded)")
+            raise ValueError(f"{name} runs on one GPU per replica (its state and pages are not sharded)")
         self.cfg, self.ac = cfg, cfg.arch_config
         self.device, self.dtype = torch.device(device), dtype
         self.tp_rank, self.tp_size = 0, 1
@@ -139,12 +139,18 @@ class HybridLM:
                 raise ValueError(f"{name}: shape {tuple(t.shape)}, the config gives {tuple(shape)}")
             w[name] = t.to(device=self.device, dtype=self.dtype if t.is_floating_point() else t.dtype).contiguous()
         for i, m in enumerate(self.mixers):
+            if self.weight_owner(i) != i:  # the layer runs another layer's tensors (and its mixer object)
+                continue
             rows = m.proj_rows()
             w[f"l{i}.mix._in"] = torch.cat([w.pop(name) for name, _ in rows]).contiguous()
             if hasattr(m, "finish_weights"):
                 m.finish_weights(w)
         self.finish_weights(w)
         self.w = w
+
+    def weight_owner(self, i: int) -> int:
+        """The layer whose tensors layer i runs: itself, unless the design lets layers share weights."""
+        return i
 
     def finish_weights(self, w: dict) -> None:
         """A design's own re-packing of its non-mixer weights."""

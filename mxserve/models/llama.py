@@ -522,4 +522,7 @@ def build_model(cfg: ModelConfig, device, dtype=torch.bfloat16, moe_dispatch: st
     if cfg.arch == "tapasun":
         from .tapasun import TapasunLM
         return TapasunLM(cfg, device, dtype, block_size)
+    if cfg.arch == "momuvik":
+        from .momuvik import MomuvikLM
+        return MomuvikLM(cfg, device, dtype, block_size)
     return TransformerLM(cfg, device, dtype, moe_dispatch)

@@ -22,6 +22,11 @@ in a slot) and computes its output from a step's flattened token batch.
                         convolutions and unit-norm q/k, per-head RMS norm and a sigmoid output gate
   ScaledPair            two mixers reading the same input, summed with fixed scales through one
                         output projection over their concatenated activations
+  LatentAttention       softmax attention whose keys and values are expansions of one normed low-rank
+                        latent per token plus one rotated key part shared by the heads (half-split
+                        rotary pairs), queries through a normed latent of their own, optional learned
+                        sink; only the latent and the rotated part are cached, the expansions are
+                        folded into the query and the output
 
 The kernels are in mxserve/ops/seqmix.py (csrc/mixers/*.hip on the GPU).
 """
@@ -454,6 +459,70 @@ class ScaledPair(Mixer):
         self.left.mix(parts[:nl], h, w, ctx, koff, voff, soff, out=buf[:, :cl], out_scale=self.ls)
         self.right.mix(parts[nl:], h, w, ctx, koff, voff, soff, out=buf[:, cl:], out_scale=self.rs)
         return ops.linear(buf, w[self.p + "_o"])
+
+
+class LatentAttention(Mixer):
+    """Per head the query and key are [dim plain | rot_dim rotated], the value has vdim entries.
+        c_q = RMSNorm(W_dq h) * w_qn,  q = W_uq c_q
+        [c | r] = W_dkv h,  c <- RMSNorm(c) * w_kvn (kv_rank entries),  r rotated (rot_dim entries, one for all heads)
+        k_h = [W_uk,h c | r],  v_h = W_uv,h c,  score = scale * q_h . k_h,  out = W_o [softmax-weighted v_h]_h
+    The pages hold the row [c | r] per token (one kv head of kv_rank + rot_dim entries); values are the
+    row's first kv_rank entries, so nothing is stored twice.  W_uk is folded into the query
+    (q'_h = [W_uk,h^T q_h,plain | q_h,rot], score = scale * q'_h . [c | r]) and W_uv is applied to the
+    weighted sum of latents: every head attends over the same rows, with head sizes kv_rank + rot_dim
+    and kv_rank.  sink: None | "learned" (tensor `<prefix>sink` [heads])."""
+
+    def __init__(self, prefix: str, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
+                 q_rank: int, scale: float, rot: dict, sink: Optional[str] = "learned"):
+        if int(rot["dims"]) != rot_dim or rot_dim % 2:
+            raise ValueError(f"{prefix}: the rotated part has rot_dim = rot.dims entries, an even number")
+        if sink not in (None, "learned"):
+            raise ValueError(f"{prefix}: unknown sink {sink!r}")
+        self.p, self.width = prefix, width
+        self.heads, self.dn, self.dr, self.vd = int(heads), int(dim), int(rot_dim), int(vdim)
+        self.rank, self.q_rank, self.scale, self.sink = int(kv_rank), int(q_rank), float(scale), sink
+        self.kv_heads, self.dk, self.dv = 1, self.rank + self.dr, 0  # the page row; values are a slice of it
+        self.freqs = rotary_frequencies(self.dr, float(rot["base"]), None)
+
+    def proj_rows(self) -> list:
+        return [(self.p + "dq", self.q_rank), (self.p + "dkv", self.rank + self.dr)]
+
+    def extra_shapes(self) -> dict:
+        p, H = self.p, self.heads
+        sh = {p + "dq.norm": (self.q_rank,), p + "dkv.norm": (self.rank,), p + "uq": (H * (self.dn + self.dr), self.q_rank),
+              p + "uk": (H * self.dn, self.rank), p + "uv": (H * self.vd, self.rank), p + "o": (self.width, H * self.vd)}
+        if self.sink == "learned":
+            sh[p + "sink"] = (H,)
+        return sh
+
+    def finish_weights(self, w: dict) -> None:
+        p, H = self.p, self.heads
+        self.freqs = self.freqs.to(w[p + "o"].device)
+        if self.sink == "learned":
+            _fp32(w, p + "sink")
+        # per-head factors of the two batched products: q'_plain = q_plain @ uk[h], out_h = latent_h @ uv[h]^T
+        w[p + "uk"] = w[p + "uk"].view(H, self.dn, self.rank).contiguous()
+        w[p + "uv"] = w[p + "uv"].view(H, self.vd, self.rank).transpose(1, 2).contiguous()
+
+    def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):
+        md, p, H = ctx.md, self.p, self.heads
+        dq, dkv = parts
+        T = h.shape[0]
+        cq = seqmix.latent_prep(dq, dkv, md.positions, md.slot_mapping, ctx.cache, koff, self.rank, ctx.block_size,
+                                self.freqs, w[p + "dq.norm"], w[p + "dkv.norm"], ctx.eps)
+        q = ops.linear(cq, w[p + "uq"])  # [T, H * (dn + dr)]
+        dq_, dk = self.dn + self.dr, self.dk
+        qf = torch.empty(T, H * dk, dtype=q.dtype, device=q.device)
+        # the plain part through W_uk^T, head by head, straight into its columns of the folded query
+        torch.bmm(q.view(T, H, dq_)[:, :, :self.dn].transpose(0, 1), w[p + "uk"],
+                  out=qf.view(T, H, dk)[:, :, :self.rank].transpose(0, 1))
+        seqmix.rope_half_into(qf, q, md.positions, H, dq_, self.dn, dk, self.rank, self.freqs)
+        lat = seqmix.window_attention(qf, ctx.cache, md.block_tables, md.query_start_loc, md.seq_lens, koff, koff, H, 1,
+                                      dk, self.rank, ctx.block_size, self.scale, 0, 0, md.max_query_len,
+                                      sink=w.get(p + "sink"), v_stride=dk)
+        o = torch.empty(T, H * self.vd, dtype=q.dtype, device=q.device)
+        torch.bmm(lat.view(T, H, self.rank).transpose(0, 1), w[p + "uv"], out=o.view(T, H, self.vd).transpose(0, 1))
+        return ops.linear(o, w[p + "o"])
 
 
 def build_mixer(kind: str, prefix: str, width: int, mc: dict) -> Mixer:

@@ -64,22 +64,24 @@ def _rms(x: torch.Tensor, eps: float) -> torch.Tensor:
 def resid_update(x: torch.Tensor, a: Optional[torch.Tensor], eps: float, *, wa: Optional[torch.Tensor] = None,
                  b: Optional[torch.Tensor] = None, wb: Optional[torch.Tensor] = None,
                  bias: Optional[torch.Tensor] = None, assign: bool = False,
-                 norm_w: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None):
+                 norm_w: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
+                 a_scale: float = 1.0, w_offset: float = 0.0):
     """One pass over the fp32 residual stream x [T, W], in place:
-        d = a                      (wa: RMSNorm(a) * wa)
+        d = a * a_scale            (wa: RMSNorm(a) * wa)
         d = (d + RMSNorm(b) * wb) / 2      when b is given (two branches, each normed over the width)
         d += bias                  (a [W] vector)
         x = d if assign else x + d
-    and, when norm_w is given, returns RMSNorm(x) * norm_w in out_dtype (the next sublayer's input).
+    and, when norm_w is given, returns RMSNorm(x) * (w_offset + norm_w) in out_dtype (the next
+    sublayer's input; w_offset = 1 for weights stored as their difference from one, added in fp32).
     a = None leaves x as it is (norm only).  All sums and norms in fp32."""
     if _gpu(x):
         h = None
         if norm_w is not None:
             h = torch.empty(x.shape, dtype=out_dtype or norm_w.dtype, device=x.device)
-        ext().resid_update(x, a, wa, b, wb, bias, bool(assign), norm_w, h, float(eps))
+        ext().resid_update(x, a, wa, b, wb, bias, bool(assign), norm_w, h, float(eps), float(a_scale), float(w_offset))
         return h
     if a is not None:
-        d = a.float()
+        d = a.float() * a_scale if a_scale != 1.0 else a.float()
         if wa is not None:
             d = _rms(d, eps) * wa.float()
         if b is not None:
@@ -92,7 +94,7 @@ def resid_update(x: torch.Tensor, a: Optional[torch.Tensor], eps: float, *, wa: 
             x.add_(d)
     if norm_w is None:
         return None
-    return (_rms(x, eps) * norm_w.float()).to(out_dtype or norm_w.dtype)
+    return (_rms(x, eps) * (norm_w.float() + w_offset if w_offset else norm_w.float())).to(out_dtype or norm_w.dtype)
 
 
 def cast_into(dst: torch.Tensor, x: torch.Tensor) -> None:
@@ -165,23 +167,31 @@ def kv_write(cache: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_mapping
 def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, qsl: torch.Tensor,
                      seq_lens: torch.Tensor, koff: int, voff: int, num_heads: int, num_kv_heads: int, dk: int,
                      dv: int, block_size: int, scale: float, window: int, keep_first: int,
-                     max_query_len: int = 0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     max_query_len: int = 0, sink: Optional[torch.Tensor] = None, v_stride: int = 0) -> torch.Tensor:
     """Softmax attention over the paged cache (this step's keys already written).  The query at
     position i sees key j <= i when i - j < window or j < keep_first (window <= 0: every j <= i).
     q [T, H*dk] (row-strided view) -> [T, H*dv] in q's dtype; scores and weights in fp32.
     Query head h reads kv head h // (H / Hkv).  sink (fp32 [H]): the softmax denominator of head h also
-    holds exp(sink[h]), a key without a value whose score is not scaled.  max_query_len: the longest chunk of the step (host
+    holds exp(sink[h]), a key without a value whose score is not scaled.  v_stride (elements, 0: dv): the
+    distance between two tokens' value rows, for values that are a slice of a wider cached row (then
+    num_kv_heads is 1 and voff points at the slice inside the first row).  max_query_len: the longest chunk of the step (host
     int); from 16 rows a bf16 step with head sizes that are multiples of 16 runs the MFMA kernel."""
     T = q.shape[0]
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
         ext().window_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), int(voff), num_heads,
                                num_kv_heads, dk, dv, block_size, float(scale), int(window), int(keep_first),
-                               int(max_query_len), sink)
+                               int(max_query_len), sink, int(v_stride))
         return out
     out = torch.zeros(T, num_heads, dv, dtype=torch.float32)
     kc = cache[:, koff:koff + num_kv_heads * block_size * dk].view(-1, num_kv_heads, block_size, dk)
-    vc = cache[:, voff:voff + num_kv_heads * block_size * dv].view(-1, num_kv_heads, block_size, dv)
+    if v_stride and v_stride != dv:
+        if num_kv_heads != 1:
+            raise ValueError("strided value rows need a single kv head")
+        vc = torch.as_strided(cache, (cache.shape[0], 1, block_size, dv), (cache.stride(0), 0, v_stride, 1),
+                              cache.storage_offset() + voff)
+    else:
+        vc = cache[:, voff:voff + num_kv_heads * block_size * dv].view(-1, num_kv_heads, block_size, dv)
     g = num_heads // num_kv_heads
     ql, sl = qsl.tolist(), seq_lens.tolist()
     for s in range(len(sl)):
@@ -567,3 +577,153 @@ def gated_norm(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, eps: float,
         y = y * gf
     out.copy_((y * out_scale).to(out.dtype))
     return out
+
+
+# ----------------------------------------------------------------------------- latent attention
+def _rotate_half(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
+    """x fp32 [T, heads, 2n]: coordinate i pairs with i + n and the pair turns by pos * freqs[i]."""
+    n = freqs.numel()
+    ang = pos.to(torch.float32).view(-1, 1, 1) * freqs.float().view(1, 1, n)
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, v = x[..., :n], x[..., n:]
+    return torch.cat([u * c - v * s, v * c + u * s], dim=-1)
+
+
+def latent_prep(dq: torch.Tensor, dkv: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor,
+                cache: torch.Tensor, koff: int, rank: int, block_size: int, freqs: torch.Tensor,
+                q_norm: torch.Tensor, kv_norm: torch.Tensor, eps: float) -> torch.Tensor:
+    """The two down-projections of a latent attention, from the fused projection to what the next
+    steps read, in one launch.  dq [T, q_rank] (row-strided view): returns RMSNorm(dq) * q_norm as a
+    new [T, q_rank].  dkv [T, rank + 2n]: the first `rank` columns RMS-normed times kv_norm, the last
+    2n (n = len(freqs)) turned in the half-split layout (i pairs with i + n) by position * freqs[i];
+    the row [latent | turned part] goes into the paged cache at `koff` as [BS, rank + 2n] (one shared
+    kv head; slot -1: not written).  Norms, angles and turns in fp32, one rounding at the end."""
+    T, qr = dq.shape
+    n = freqs.numel()
+    dk = rank + 2 * n
+    if _gpu(dq):
+        cq = torch.empty(T, qr, dtype=dq.dtype, device=dq.device)
+        ext().latent_prep(cq, dq, dkv, positions, slot_mapping, cache, int(koff), int(rank), int(block_size), freqs,
+                          q_norm, kv_norm, float(eps))
+        return cq
+    cq = (_rms(dq.float(), eps) * q_norm.float()).to(dq.dtype)
+    d = dkv.float()
+    c = _rms(d[:, :rank], eps) * kv_norm.float()
+    kr = _rotate_half(d[:, rank:].unsqueeze(1), positions, freqs).squeeze(1)
+    row = torch.cat([c, kr], dim=-1).to(cache.dtype)
+    ok = slot_mapping >= 0
+    slots = slot_mapping[ok]
+    kc = cache[:, koff:koff + block_size * dk].view(-1, block_size, dk)
+    kc[slots // block_size, slots % block_size] = row[ok]
+    return cq
+
+
+def rope_half_into(out: torch.Tensor, x: torch.Tensor, positions: torch.Tensor, heads: int, x_dim: int, x_col: int,
+                   out_dim: int, out_col: int, freqs: torch.Tensor) -> None:
+    """Per token and head: the 2n columns of x's head (x [T, heads*x_dim], from column x_col of the head)
+    turned in the half-split layout by position * freqs[i], written to columns out_col.. of the same
+    head in out [T, heads*out_dim].  fp32 inside."""
+    n = freqs.numel()
+    if _gpu(x):
+        ext().rope_half_into(out, x, positions, int(heads), int(x_dim), int(x_col), int(out_dim), int(out_col), freqs)
+        return
+    T = x.shape[0]
+    part = x.reshape(T, heads, x_dim)[:, :, x_col:x_col + 2 * n].float()
+    out.view(T, heads, out_dim)[:, :, out_col:out_col + 2 * n] = _rotate_half(part, positions, freqs).to(out.dtype)
+
+
+# ----------------------------------------------------------------------------- routed experts
+def route_topk(logits: torch.Tensor, k: int, renorm: bool = False) -> tuple:
+    """Sigmoid router: scores = sigmoid(logits) (fp32 [T, E]); the k largest per token (ties: the
+    lower index first), their scores as weights (renorm: divided by their sum).
+    -> (weights fp32 [T, k], ids int32 [T, k])."""
+    T, E = logits.shape
+    if _gpu(logits):
+        w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+        ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+        ext().route_topk(w, ids, logits, bool(renorm))
+        return w, ids
+    s = torch.sigmoid(logits.float())
+    order = torch.argsort(s, dim=-1, descending=True, stable=True)[:, :k]
+    w = torch.gather(s, 1, order)
+    if renorm:
+        w = w / w.sum(-1, keepdim=True)
+    return w, order.to(torch.int32)
+
+
+def capped_glu(gu: torch.Tensor, limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """A fused [gate | up] projection [R, 2F] -> [R, F]:  g = min(gate, limit), u = clamp(up, -limit, limit),
+    g * sigmoid(alpha * g) * (u + 1); fp32 inside."""
+    Fh = gu.shape[1] // 2
+    if _gpu(gu):
+        out = torch.empty(gu.shape[0], Fh, dtype=gu.dtype, device=gu.device)
+        ext().capped_glu(out, gu, float(limit), float(alpha))
+        return out
+    g = gu[:, :Fh].float().clamp(max=limit)
+    u = gu[:, Fh:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+
+
+def expert_align(ids: torch.Tensor, num_experts: int) -> tuple:
+    """Counting sort of the (token, slot) pairs by expert.  ids int32 [T, k] -> (offs int32 [E + 1]:
+    expert e owns the sorted rows offs[e]:offs[e+1]; inv int32 [T*k]: the sorted row of pair p = t*k + j;
+    the order of one expert's rows is free)."""
+    T, k = ids.shape
+    if _gpu(ids):
+        offs = torch.empty(num_experts + 1, dtype=torch.int32, device=ids.device)
+        inv = torch.empty(T * k, dtype=torch.int32, device=ids.device)
+        ext().expert_align(offs, inv, ids, int(num_experts))
+        return offs, inv
+    flat = ids.reshape(-1).long()
+    order = torch.argsort(flat, stable=True)
+    inv = torch.empty_like(order)
+    inv[order] = torch.arange(order.numel())
+    counts = torch.bincount(flat, minlength=num_experts)
+    offs = torch.cat([torch.zeros(1, dtype=torch.long), counts.cumsum(0)])
+    return offs.to(torch.int32), inv.to(torch.int32)
+
+
+def gather_scaled(h: torch.Tensor, weights: torch.Tensor, inv: torch.Tensor) -> torch.Tensor:
+    """xs[inv[p]] = weights[p] * h[p // k] for every pair p (weights fp32 [T, k]): the experts' inputs,
+    sorted by expert, each already times its routing weight (product in fp32, rounded once)."""
+    T, k = weights.shape
+    xs = torch.empty(T * k, h.shape[1], dtype=h.dtype, device=h.device)
+    if _gpu(h):
+        ext().gather_scaled(xs, h, weights, inv)
+        return xs
+    rows = (h.float().unsqueeze(1) * weights.float().unsqueeze(2)).reshape(T * k, -1).to(h.dtype)
+    xs[inv.long()] = rows
+    return xs
+
+
+def spread_scaled(h: torch.Tensor, weights: torch.Tensor, ids: torch.Tensor, num_experts: int) -> torch.Tensor:
+    """[E, T, W]: row (e, t) = weights[t, j] * h[t] where ids[t, j] = e, zeros for the experts a token
+    did not choose (the experts' inputs for a batched product over all experts, no sorting)."""
+    T, k = weights.shape
+    if _gpu(h):
+        xs = torch.empty(num_experts, T, h.shape[1], dtype=h.dtype, device=h.device)
+        ext().spread_scaled(xs, h, weights, ids)
+        return xs
+    cw = torch.zeros(T, num_experts, dtype=torch.float32)
+    cw.scatter_(1, ids.long(), weights.float())
+    return (cw.t().unsqueeze(2) * h.float().unsqueeze(0)).to(h.dtype)
+
+
+def expert_combine(ys: torch.Tensor, index: Optional[torch.Tensor], k: int, T: int, extra: Optional[torch.Tensor] = None,
+                   row_stride: int = 0) -> torch.Tensor:
+    """out[t] = sum_j ys[index[t*k + j]] (+ extra[t]); index None: row j*row_stride + t (the k slabs
+    of a [k, T, W] stack).  Summed in fp32, rounded once."""
+    W = ys.shape[-1]
+    y2 = ys.reshape(-1, W)
+    if _gpu(ys):
+        out = torch.empty(T, W, dtype=ys.dtype, device=ys.device)
+        ext().expert_combine(out, y2, index, int(k), extra, int(row_stride))
+        return out
+    if index is None:
+        idx = (torch.arange(k).view(1, k) * row_stride + torch.arange(T).view(T, 1)).reshape(-1)
+    else:
+        idx = index.long()
+    acc = y2[idx].float().view(T, k, W).sum(1)
+    if extra is not None:
+        acc = acc + extra.float()
+    return acc.to(ys.dtype)
