@@ -118,18 +118,25 @@ class Oracle:
         self.eps = float(cfg["norm"]["eps"])
         self.m = float(cfg.get("residual_mult", 1.0))
         self.escale = float((cfg.get("embedding") or {}).get("scale", 1.0))
-        self.src = [int(l.get("weights_of", i)) for i, l in enumerate(cfg["layers"])]
+        self.src = []  # the layer whose tensors layer i runs (a named layer may itself name another)
+        for i in range(len(cfg["layers"])):
+            j = i
+            while cfg["layers"][j].get("weights_of") is not None:
+                j = int(cfg["layers"][j]["weights_of"])
+            self.src.append(j)
         self.mixers = []
         for i, l in enumerate(cfg["layers"]):
             if l["type"] != "latent_attention":
                 raise ValueError(l["type"])
             self.mixers.append(LatentAttention(l["mixer"], w, f"l{self.src[i]}.mix.", self.eps))
         self.pos = 0
+        # per token: the smallest gap, over its routed layers, between the last chosen score and the best one left out
+        self.margins = []
 
     def step(self, token: int):
         w, eps, m = self.w, self.eps, self.m
         x = w["embed"][token] * self.escale
-        streams = []
+        streams, margin = [], math.inf
         for i, l in enumerate(self.cfg["layers"]):
             p = f"l{self.src[i]}."
             x = x + m * self.mixers[i].step(offset_norm(x, w[p + "norm1"], eps), self.pos)
@@ -139,20 +146,28 @@ class Oracle:
                 if mlp.get("kind", "dense") == "dense":
                     y = dense_ff(h, w, p + "mlp.")
                 else:
-                    y, _ = routed_ff(h, w, p + "mlp.", mlp)
+                    y, sc = routed_ff(h, w, p + "mlp.", mlp)
+                    top = int(mlp["router"]["top"])
+                    if top < len(sc):
+                        srt = np.sort(sc)[::-1]
+                        margin = min(margin, float(srt[top - 1] - srt[top]))
                 x = x + m * y
             streams.append(x.copy())
         self.pos += 1
+        self.margins.append(margin)
         logits = w["embed"] @ offset_norm(x, w["final.norm"], eps)
         return logits, streams
 
 
-def run(cfg: dict, w: dict, tokens) -> tuple:
-    """(logits [n, vocab], streams [layers, n, width]) of one sequence."""
+def run(cfg: dict, w: dict, tokens, margins=None) -> tuple:
+    """(logits [n, vocab], streams [layers, n, width]) of one sequence; a list passed as `margins`
+    receives every token's routing margin."""
     o = Oracle(cfg, w)
     lg, st = [], []
     for t in tokens:
         a, b = o.step(int(t))
         lg.append(a)
         st.append(b)
+    if margins is not None:
+        margins.extend(o.margins)
     return np.stack(lg), np.stack([np.stack(s) for s in st]).transpose(1, 0, 2)
