@@ -35,6 +35,8 @@ void launch_causal_conv(void*, const void*, long, const void*, const void*, floa
 void launch_gated_norm(void*, long, const float*, const void*, long, const void*, int, int, int, int, float, int, int,
                        float, bool, hipStream_t);
 bool launch_column_scan(const ScanArgs&, int, bool, bool, hipStream_t);
+bool launch_latent_attention(void*, float*, const void*, long, const void*, long, const int*, int, const int*, const int*,
+                             int, int, int, int, int, int, int, float, int, const float*, int, hipStream_t);
 void launch_latent_prep(void*, const void*, long, const void*, long, const int64_t*, const int64_t*, void*, long, int, int,
                         int, int, int, int, const float*, const void*, const void*, float, bool, hipStream_t);
 void launch_rope_half_into(void*, long, const void*, long, const int64_t*, int, int, int, int, int, int, const float*, int,
@@ -456,6 +458,37 @@ void latent_prep(at::Tensor cq, at::Tensor dq, at::Tensor dkv, at::Tensor positi
                           static_cast<float>(eps), bf, stream());
 }
 
+// The matrix-core latent attention (bf16).  Returns false when the sizes are not the kernel's: nothing
+// was launched and the caller runs window_attention with strided value rows instead.
+bool latent_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor block_tables, at::Tensor qsl,
+                      at::Tensor seq_lens, int64_t koff, int64_t H, int64_t dk, int64_t rank, int64_t bs, double scale,
+                      int64_t max_query_len, OptT sink, int64_t nsplit, OptT part) {
+  if (!is_bf(q)) return false;
+  const float* sinkp = nullptr;
+  if (sink.has_value()) {
+    sinkp = f32(*sink, "sink");
+    TORCH_CHECK(sink->numel() == H, "sink: fp32 [H]");
+  }
+  const int64_t T = q.size(0), S = seq_lens.numel();
+  TORCH_CHECK(rank >= 1 && rank <= dk && H >= 1, "1 <= rank <= dk");
+  check_cache(cache, true, koff, koff, 1, dk, 0, bs);
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == H * rank &&
+              is_bf(out), "out: bf16 [T, H*rank]");
+  TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == at::kInt && block_tables.dim() == 2 &&
+              block_tables.size(0) >= S && block_tables.stride(1) == 1, "block_tables: int32 [S, max_blocks]");
+  float* pp = nullptr;
+  if (nsplit > 1) {
+    TORCH_CHECK(part.has_value() && part->numel() >= T * H * nsplit * (rank + 4), "part: fp32 [T*H, nsplit, rank + 4]");
+    pp = f32(*part, "part");
+  }
+  return mxs::launch_latent_attention(
+      out.data_ptr(), pp, mat(q, true, T, H * dk, "q"), q.stride(0), cache.data_ptr(), cache.stride(0),
+      block_tables.data_ptr<int>(), static_cast<int>(block_tables.stride(0)), i32(qsl, S + 1, "qsl"),
+      i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(koff), static_cast<int>(H),
+      static_cast<int>(dk), static_cast<int>(rank), static_cast<int>(bs), static_cast<float>(scale),
+      static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(max_query_len, T))), sinkp, static_cast<int>(nsplit), stream());
+}
+
 void rope_half_into(at::Tensor out, at::Tensor x, at::Tensor positions, int64_t heads, int64_t x_dim, int64_t x_col,
                     int64_t out_dim, int64_t out_col, at::Tensor freqs) {
   const bool bf = is_bf(x);
@@ -562,6 +595,7 @@ PYBIND11_MODULE(_M, m) {
   m.def("delta_scan", &delta_scan);
   m.def("latent_prep", &latent_prep);
   m.def("rope_half_into", &rope_half_into);
+  m.def("latent_attention", &latent_attention);
   m.def("route_topk", &route_topk);
   m.def("capped_glu", &capped_glu);
   m.def("expert_align", &expert_align);

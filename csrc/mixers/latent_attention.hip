@@ -1,0 +1,263 @@
+// Latent attention on the matrix cores (gfx950, bf16): every query head attends over the same
+// cached rows [latent (rank) | rotated key part], dk entries a row, and the values are the rows'
+// first `rank` entries.  Prompt chunks and single decoded tokens run the same kernel.
+//
+// The rows of a sequence's step are its (token, head) pairs, flattened; a wave owns 16 consecutive
+// rows and walks the 16-key cache blocks that its rows see (causal), or one of `nsplit` stretches of
+// them.  No workgroup barriers: the four waves of a workgroup are independent.  Per block, with
+// v_mfma_f32_16x16x16_bf16:
+//   S^T = K Q^T      A = the block's 16 key rows, loaded from the pages as 16-byte pieces that are
+//                    used as they are: lane (key c, group kg) holds entries 32 kk + 8 kg .. + 7 of its
+//                    key, the two halves of a piece feed two MFMAs, and Q^T (held in registers for
+//                    the whole walk) is loaded in the same order, so the products pair up whatever
+//                    the order of the summed index is.  The accumulator has the row on the lane
+//                    and 4 keys per lane: maxima and sums are per-lane work plus two lane exchanges.
+//   O^T += V^T P^T   B = P^T straight from the S^T accumulator's registers, every weight split into
+//                    two bf16 halves (p = hi + lo, two MFMAs) so that the product keeps 16 mantissa
+//                    bits of the fp32 weight.  A = V^T: the same registers that held the key pieces
+//                    are written into the wave's LDS area transposed ([entry][key], 2-byte stores)
+//                    and read back key-contiguous with one 8-byte load per tile.
+// The next block's pieces are loaded while the values are multiplied.  Scores (log2 units), maxima,
+// sums and the output accumulator are fp32.  A sink (fp32 [H], optional) starts the running maximum at
+// sink[h] and the running sum at 1.  With nsplit > 1 a wave writes its stretch's (maximum, sum,
+// unnormalised output) and latent_attention_combine merges the stretches of a row.
+#include "mix_common.h"
+
+namespace mxs {
+
+typedef short s4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kVtPitch = 20;  // bf16 per transposed row: 16 keys + 4, so that the four key groups fall into different banks
+
+__device__ __forceinline__ s4_t lo4(const uint4& a) {
+  union { uint2 u; s4_t s; } x;
+  x.u = make_uint2(a.x, a.y);
+  return x.s;
+}
+__device__ __forceinline__ s4_t hi4(const uint4& a) {
+  union { uint2 u; s4_t s; } x;
+  x.u = make_uint2(a.z, a.w);
+  return x.s;
+}
+
+constexpr int kPartHead = 4;  // floats ahead of a stretch's output: maximum, sum, two unused (16-byte rows)
+
+// KKM: 32-entry chunks of a row (dk <= 32 KKM); VTM: 16-entry value tiles (rank <= 16 VTM); NW: waves of
+// a workgroup (its LDS is NW transposed value blocks)
+template <int KKM, int VTM, int NW>
+__global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
+    bf16_t* __restrict__ out, float* __restrict__ part, const bf16_t* __restrict__ q, long q_stride,
+    const bf16_t* __restrict__ cache, long block_stride, const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ qsl, const int* __restrict__ seq_lens, int koff, int H, int dk, int rank, float scale,
+    const float* __restrict__ sink, int nsplit) {
+  extern __shared__ __attribute__((aligned(16))) bf16_t vt_lds[];  // [NW waves][16 VTM entries][kVtPitch]
+  const int s = blockIdx.z;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  bf16_t* vt_w = vt_lds + wid * (16 * VTM * kVtPitch);
+  const int row0 = qsl[s], qlen = qsl[s + 1] - row0;
+  const int nrows = qlen * H;
+  const int id = blockIdx.x * NW + wid;
+  const int tile = id / nsplit, sp = id - tile * nsplit;
+  if (tile * 16 >= nrows) return;  // wave-uniform (no workgroup barrier is used below)
+  const int c = lane & 15, kg = lane >> 4;
+  const int r = tile * 16 + c;
+  const bool rok = r < nrows;
+  const int rr = rok ? r : nrows - 1;
+  const int tok = rr / H, hd = rr - tok * H;
+  // positions, kept inside the block table whatever the metadata says
+  const int last = bt_stride * 16 - 1;
+  const int base = max(seq_lens[s] - qlen, 0);
+  const int pq = min(base + tok, last);
+  const int p_first = min(base + (tile * 16) / H, last);
+  const int p_last = min(base + min(tile * 16 + 15, nrows - 1) / H, last);
+  const int nblk = (p_last >> 4) + 1;
+  const int b0 = static_cast<int>(static_cast<long>(nblk) * sp / nsplit);
+  const int b1 = static_cast<int>(static_cast<long>(nblk) * (sp + 1) / nsplit);
+  const int KK = (dk + 31) >> 5, VT = rank >> 4;
+  const int* bt = block_tables + static_cast<long>(s) * bt_stride;
+  uint4 qf[KKM];
+  {
+    const bf16_t* qp = q + static_cast<long>(row0 + tok) * q_stride + static_cast<long>(hd) * dk + 8 * kg;
+#pragma unroll
+    for (int kk = 0; kk < KKM; ++kk)
+      qf[kk] = (kk < KK && rok && 32 * kk + 8 * kg + 8 <= dk) ? *reinterpret_cast<const uint4*>(qp + 32 * kk)
+                                                              : make_uint4(0, 0, 0, 0);
+  }
+  const float L2E = 1.4426950408889634f;
+  float m = (sink && sp == 0) ? sink[hd] * L2E : -INFINITY;
+  float l = (sink && sp == 0 && kg == 0) ? 1.f : 0.f;  // a lane's share of its row's sum (its key group's)
+  f4_t o[VTM];
+#pragma unroll
+  for (int vt = 0; vt < VTM; ++vt) o[vt] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const float sl2 = scale * L2E;
+  uint4 kr[KKM];
+  auto load_block = [&](int kb) {
+    const bf16_t* kp = cache + static_cast<long>(bt[kb]) * block_stride + koff + static_cast<long>(c) * dk + 8 * kg;
+#pragma unroll
+    for (int kk = 0; kk < KKM; ++kk)
+      kr[kk] = (kk < KK && 32 * kk + 8 * kg + 8 <= dk) ? *reinterpret_cast<const uint4*>(kp + 32 * kk)
+                                                       : make_uint4(0, 0, 0, 0);
+  };
+  if (b0 < b1) load_block(b0);
+  for (int kb = b0; kb < b1; ++kb) {
+    const int k0 = kb * 16;
+    f4_t acc = f4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int kk = 0; kk < KKM; ++kk) {
+      if (kk < KK) {
+        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(lo4(kr[kk]), lo4(qf[kk]), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(hi4(kr[kk]), hi4(qf[kk]), acc, 0, 0, 0);
+      }
+    }
+    // the block's values, transposed, into the wave's LDS area; rows past the tile's last position
+    // may hold anything (also NaN): they are written as zeros
+    __builtin_amdgcn_wave_barrier();  // the previous block's reads come first
+    {
+      const bool kok = k0 + c <= p_last;
+#pragma unroll
+      for (int kk = 0; kk < KKM; ++kk) {
+        const int d0 = 32 * kk + 8 * kg;
+        if (kk < KK && d0 < rank) {
+          const uint4 a = kok ? kr[kk] : make_uint4(0, 0, 0, 0);
+          bf16_t* w = vt_w + d0 * kVtPitch + c;
+          w[0] = static_cast<bf16_t>(a.x & 0xFFFFu);
+          w[kVtPitch] = static_cast<bf16_t>(a.x >> 16);
+          w[2 * kVtPitch] = static_cast<bf16_t>(a.y & 0xFFFFu);
+          w[3 * kVtPitch] = static_cast<bf16_t>(a.y >> 16);
+          w[4 * kVtPitch] = static_cast<bf16_t>(a.z & 0xFFFFu);
+          w[5 * kVtPitch] = static_cast<bf16_t>(a.z >> 16);
+          w[6 * kVtPitch] = static_cast<bf16_t>(a.w & 0xFFFFu);
+          w[7 * kVtPitch] = static_cast<bf16_t>(a.w >> 16);
+        }
+      }
+    }
+    if (kb + 1 < b1) load_block(kb + 1);  // in flight while the weights are made and the values multiplied
+    // a block that every row of the tile sees whole needs no mask
+    const bool whole = k0 + 15 <= p_first;
+    float sv[4], mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (whole) {
+        sv[i] = acc[i] * sl2;
+      } else {
+        const int j = k0 + 4 * kg + i;
+        sv[i] = (rok && j <= pq) ? acc[i] * sl2 : -INFINITY;
+      }
+      mx = fmaxf(mx, sv[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {  // rescale only when some row's maximum moved
+      const float corr = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+      l *= corr;
+#pragma unroll
+      for (int vt = 0; vt < VTM; ++vt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[vt][i] *= corr;
+      m = m_new;
+    }
+    s4_t ph, pl;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      // a row with nothing visible yet (m = -inf) must not turn -inf - -inf into a weight
+      const float pr = (whole || sv[i] != -INFINITY) ? __builtin_amdgcn_exp2f(sv[i] - m) : 0.f;
+      l += pr;
+      // pr = hi + lo: hi the upper 16 bits (exact), lo = pr - hi rounded to bf16 (pr >= 0, finite)
+      const uint32_t u = __float_as_uint(pr), uh = u & 0xFFFF0000u;
+      uint32_t ul = __float_as_uint(pr - __uint_as_float(uh));
+      ul += 0x7FFFu + ((ul >> 16) & 1u);
+      ph[i] = static_cast<short>(uh >> 16);
+      pl[i] = static_cast<short>(ul >> 16);
+    }
+    __builtin_amdgcn_wave_barrier();
+    const bf16_t* vp = vt_w + c * kVtPitch + 4 * kg;
+#pragma unroll
+    for (int vt = 0; vt < VTM; ++vt) {
+      if (vt < VT) {
+        const s4_t a = *reinterpret_cast<const s4_t*>(vp + 16 * vt * kVtPitch);
+        const f4_t t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, o[vt], 0, 0, 0);
+        o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, t, 0, 0, 0);
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!rok) return;
+  const long grow = static_cast<long>(row0 + tok) * H + hd;  // the row among all (token, head) pairs of the step
+  if (nsplit == 1) {
+    const float inv = 1.f / l;
+    bf16_t* op = out + grow * rank + 4 * kg;
+#pragma unroll
+    for (int vt = 0; vt < VTM; ++vt) {
+      if (vt < VT) {
+        uint2 w;
+        w.x = pack2(o[vt][0] * inv, o[vt][1] * inv);
+        w.y = pack2(o[vt][2] * inv, o[vt][3] * inv);
+        *reinterpret_cast<uint2*>(op + 16 * vt) = w;
+      }
+    }
+  } else {
+    float* pp = part + (grow * nsplit + sp) * (rank + kPartHead);
+    if (kg == 0) { pp[0] = m; pp[1] = l; }
+#pragma unroll
+    for (int vt = 0; vt < VTM; ++vt)
+      if (vt < VT) *reinterpret_cast<f4_t*>(pp + kPartHead + 16 * vt + 4 * kg) = o[vt];
+  }
+}
+
+// One workgroup per (token, head) row: the stretches' (m, l, o) merged.  m is in log2 units.
+__global__ void __launch_bounds__(128) latent_attention_combine_kernel(bf16_t* __restrict__ out,
+                                                                       const float* __restrict__ part, int nsplit,
+                                                                       int rank) {
+  const long row = blockIdx.x;
+  const int ps = rank + kPartHead;
+  const float* pp = part + row * nsplit * ps;
+  float M = -INFINITY;
+  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, pp[s * ps]);
+  float L = 0.f;
+  for (int s = 0; s < nsplit; ++s) {
+    const float ms = pp[s * ps];
+    if (ms != -INFINITY) L += pp[s * ps + 1] * __builtin_amdgcn_exp2f(ms - M);
+  }
+  const float inv = 1.f / L;
+  for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      const float ms = pp[s * ps];
+      if (ms != -INFINITY) a += pp[s * ps + kPartHead + d] * __builtin_amdgcn_exp2f(ms - M);
+    }
+    out[row * rank + d] = f2bf(a * inv);
+  }
+}
+
+// False: sizes the kernel does not take (the caller runs the general kernel).
+bool launch_latent_attention(void* out, float* part, const void* q, long q_stride, const void* cache, long block_stride,
+                             const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S, int rows,
+                             int koff, int H, int dk, int rank, int bs, float scale, int max_q, const float* sink,
+                             int nsplit, hipStream_t st) {
+  if (rows == 0 || S == 0) return true;
+  if (bs != 16 || dk % 8 || rank % 16 || rank > dk || dk > 576 || rank > 512 || q_stride % 8 || koff % 8 ||
+      block_stride % 8 || reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(cache) % 16 ||
+      reinterpret_cast<uintptr_t>(part) % 16 || nsplit < 1 || (nsplit > 1 && part == nullptr))
+    return false;
+  const int tiles = (max_q * H + 15) / 16;
+#define MIX_LA(KKM, VTM, NW)                                                                                          \
+  hipLaunchKernelGGL((latent_attention_mfma_kernel<KKM, VTM, NW>), dim3((tiles * nsplit + NW - 1) / NW, 1, S),        \
+                     dim3(64 * NW), NW * 16 * VTM * kVtPitch * sizeof(bf16_t), st, (bf16_t*)out, part,                \
+                     (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl,    \
+                     seq_lens, koff, H, dk, rank, scale, sink, nsplit)
+  if (dk <= 192 && rank <= 128) MIX_LA(6, 8, 4);
+  else if (dk <= 320 && rank <= 256) MIX_LA(10, 16, 4);
+  else MIX_LA(18, 32, 2);  // 40 KB of LDS for two waves
+#undef MIX_LA
+  MXS_CHECK_LAUNCH();
+  if (nsplit > 1) {
+    hipLaunchKernelGGL(latent_attention_combine_kernel, dim3(rows * H), dim3(128), 0, st, (bf16_t*)out, part, nsplit, rank);
+    MXS_CHECK_LAUNCH();
+  }
+  return true;
+}
+
+}  // namespace mxs

@@ -517,9 +517,9 @@ class LatentAttention(Mixer):
         torch.bmm(q.view(T, H, dq_)[:, :, :self.dn].transpose(0, 1), w[p + "uk"],
                   out=qf.view(T, H, dk)[:, :, :self.rank].transpose(0, 1))
         seqmix.rope_half_into(qf, q, md.positions, H, dq_, self.dn, dk, self.rank, self.freqs)
-        lat = seqmix.window_attention(qf, ctx.cache, md.block_tables, md.query_start_loc, md.seq_lens, koff, koff, H, 1,
-                                      dk, self.rank, ctx.block_size, self.scale, 0, 0, md.max_query_len,
-                                      sink=w.get(p + "sink"), v_stride=dk)
+        lat = seqmix.latent_attention(qf, ctx.cache, md.block_tables, md.query_start_loc, md.seq_lens, koff, H, dk,
+                                      self.rank, ctx.block_size, self.scale, md.max_query_len,
+                                      getattr(md, "max_seq_len", 0), sink=w.get(p + "sink"))
         o = torch.empty(T, H * self.vd, dtype=q.dtype, device=q.device)
         torch.bmm(lat.view(T, H, self.rank).transpose(0, 1), w[p + "uv"], out=o.view(T, H, self.vd).transpose(0, 1))
         return ops.linear(o, w[p + "o"])

@@ -632,6 +632,36 @@ def rope_half_into(out: torch.Tensor, x: torch.Tensor, positions: torch.Tensor, 
     out.view(T, heads, out_dim)[:, :, out_col:out_col + 2 * n] = _rotate_half(part, positions, freqs).to(out.dtype)
 
 
+LATENT_TARGET_WAVES = 1024  # waves that fill the 256 CUs one deep: single-token steps split their keys up to this
+
+
+def latent_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, qsl: torch.Tensor,
+                     seq_lens: torch.Tensor, koff: int, num_heads: int, dk: int, rank: int, block_size: int, scale: float,
+                     max_query_len: int = 0, max_seq_len: int = 0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Softmax attention of every head over the same cached rows [latent | rotated part] (dk entries a
+    row at `koff`, written by latent_prep), causal; the values are the rows' first `rank` entries.
+    q [T, H*dk] (the folded queries) -> the weighted latents [T, H*rank]; scores and weights fp32; sink as
+    in window_attention.  bf16 on the GPU with dk a multiple of 8 up to 576 and rank a multiple of 16 up
+    to 512 runs the matrix-core kernel; a step of few rows splits each row's keys over several waves
+    (max_seq_len bounds how many are worth it) and merges the stretches.  Everything else runs
+    window_attention with one kv head and value rows dk apart."""
+    T = q.shape[0]
+    if _gpu(q) and q.dtype == torch.bfloat16 and T:
+        S = seq_lens.numel()
+        mq = max(1, min(int(max_query_len) or T, T))
+        tiles = S * (-(-mq * num_heads // 16))
+        blocks = max(1, -(-(int(max_seq_len) or 16) // 16))
+        nsplit = max(1, min(16, LATENT_TARGET_WAVES // max(tiles, 1), blocks // 2))
+        out = torch.empty(T, num_heads * rank, dtype=q.dtype, device=q.device)
+        part = (torch.empty(T * num_heads * nsplit * (rank + 4), dtype=torch.float32, device=q.device)
+                if nsplit > 1 else None)
+        if ext().latent_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), num_heads, dk, rank, block_size,
+                                  float(scale), mq, sink, nsplit, part):
+            return out
+    return window_attention(q, cache, block_tables, qsl, seq_lens, koff, koff, num_heads, 1, dk, rank, block_size, scale,
+                            0, 0, max_query_len, sink=sink, v_stride=dk)
+
+
 # ----------------------------------------------------------------------------- routed experts
 def route_topk(logits: torch.Tensor, k: int, renorm: bool = False) -> tuple:
     """Sigmoid router: scores = sigmoid(logits) (fp32 [T, E]); the k largest per token (ties: the

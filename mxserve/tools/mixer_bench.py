@@ -1,9 +1,10 @@
-"""Prefill and decode throughput of a layer-list design (Voletar, Tapasun) beside the models closest
-to it at equal width, depth and feed-forward size (random weights), through the same engine path:
-forced steps of the scheduler, the model runner, paged K/V and state slots, decode through the
-captured graphs.  Voletar stands beside a Llama-shaped model; Tapasun beside Voletar and that model.
+"""Prefill and decode throughput of a layer-list design (Voletar, Tapasun, Momuvik) beside the models
+closest to it at equal width, depth and feed-forward size (random weights), through the same engine
+path: forced steps of the scheduler, the model runner, paged K/V and state slots, decode through the
+captured graphs.  Voletar stands beside a Llama-shaped model; Tapasun beside Voletar and that model;
+Momuvik beside a Mixtral-shaped model (softmax attention and routed experts of the same sizes).
 
-  python bench.py --mixer-bench [--mixer-design voletar|tapasun] [--mixer-sizes 1024,2048]
+  python bench.py --mixer-bench [--mixer-design voletar|tapasun|momuvik] [--mixer-sizes 1024,2048]
                   [--mixer-prompt 4096] [--mixer-batch 64]
 
 Prints one JSON line per (size, model): prefill tokens/s of one prompt in one step, decode tokens/s
@@ -63,7 +64,32 @@ def tapasun_shape(width: int, layers: int = 4) -> dict:
             "layers": [kinds[i % 4] for i in range(layers)]}
 
 
+MOE_EXPERTS, MOE_TOP = 8, 2
+
+
+def momuvik_shape(width: int, layers: int = 4) -> dict:
+    """Latent attention with 128 + 64 wide query/key heads, 128-wide values and a 512-wide latent; eight
+    experts of 4/3 width, two per token, and a shared expert of a third of the width."""
+    ff = (4 * width // 3) // 256 * 256
+    att = {"heads": width // 128, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": max(3 * width // 8, 256),
+           "scale": 192 ** -0.5, "rot": {"dims": 64, "base": 10000.0}}
+    mlp = {"kind": "moe", "router": {"experts": MOE_EXPERTS, "top": MOE_TOP}, "expert": {"ff": ff, "limit": 7.0},
+           "shared": {"ff": max(width // 3 // 128 * 128, 128), "limit": 7.0}}
+    return {"architecture": "Momuvik", "width": width, "vocab": 32000, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "residual_mult": 1.0, "layers": [{"type": "latent_attention", "mixer": att, "mlp": mlp} for _ in range(layers)]}
+
+
 def register(width: int, layers: int, design: str = "voletar") -> tuple:
+    if design == "momuvik":
+        m = mcfg.momuvik_config(f"momuvik-w{width}", momuvik_shape(width, layers))
+        mcfg.REGISTRY[m.name.lower()] = m
+        base = mcfg.REGISTRY["small-llama"]
+        x = dataclasses.replace(base, name=f"mixtral-w{width}", arch="mixtral", hidden_size=width,
+                                intermediate_size=(4 * width // 3) // 256 * 256, num_layers=layers, num_heads=width // 128,
+                                num_kv_heads=max(width // 512, 1), head_dim=128, vocab_size=32000, tie_word_embeddings=False,
+                                num_experts=MOE_EXPERTS, num_experts_per_tok=MOE_TOP)
+        mcfg.REGISTRY[x.name.lower()] = x
+        return (m.name, x.name)
     if design == "tapasun":
         t = mcfg.tapasun_config(f"tapasun-w{width}", tapasun_shape(width, layers))
         mcfg.REGISTRY[t.name.lower()] = t
@@ -265,9 +291,93 @@ def tapasun_rooflines(width: int, prompt: int, batch: int, context: int) -> list
     return out
 
 
+def momuvik_rooflines(width: int, prompt: int, batch: int, context: int) -> list:
+    """Momuvik's own kernels alone, at the sizes of momuvik_shape(width): time over roofline time, each
+    beside the like kernel of the Mixtral-shaped model (its paged attention, its routed experts)."""
+    from .. import ops
+    from ..models.feedforward import RoutedExperts
+    from ..models.mixers import rotary_frequencies
+    from ..ops import moe as moe_ops
+    from ..ops import seqmix
+    dev = torch.device("cuda")
+    dt = torch.bfloat16
+    bs, out = 16, []
+    i32 = dict(dtype=torch.int32, device=dev)
+    rnd = lambda *sh: torch.randn(*sh, device=dev).to(dt)  # noqa: E731
+
+    def entry(name, t, flops, peak, bytes_, note):
+        roof = max(flops / peak, bytes_ / PEAK_HBM)
+        out.append({"kernel": name, "width": width, "ms": round(1e3 * t, 4), "roofline_ms": round(1e3 * roof, 4),
+                    "x_roofline": round(t / roof, 1), "counts": note})
+
+    shape = momuvik_shape(width)["layers"][0]
+    mc, mlp = shape["mixer"], shape["mlp"]
+    H, rank, dr, qr = mc["heads"], mc["kv_rank"], mc["rot_dim"], mc["q_rank"]
+    dk = rank + dr
+    E, top, ff = MOE_EXPERTS, MOE_TOP, mlp["expert"]["ff"]
+    for mode, T, S, ctx in (("prefill", prompt, 1, prompt), ("decode", batch, batch, context)):
+        qsl = torch.arange(0, T + 1, T // S, **i32)
+        seq = torch.full((S,), ctx, **i32)
+        nb = -(-ctx // bs)
+        bt = torch.arange(S * nb, **i32).view(S, nb)
+        pos = torch.cat([torch.arange(ctx - T // S, ctx, device=dev) for _ in range(S)])
+        slots = torch.cat([bt[s_].long().repeat_interleave(bs)[ctx - T // S:ctx] * bs + pos[:T // S] % bs for s_ in range(S)])
+        keys = ctx if mode == "decode" else ctx / 2
+        # latent attention: every head over the same rows [latent | rotated part]; values are the latent
+        cache = rnd(S * nb, bs * dk)
+        q = rnd(T, H * dk)
+        sink = torch.zeros(H, device=dev)
+        t = _time(lambda: seqmix.latent_attention(q, cache, bt, qsl, seq, 0, H, dk, rank, bs, 0.07, T // S, ctx, sink=sink), 5)
+        entry(f"latent_attention/{mode}", t, 2.0 * T * H * keys * (dk + rank), PEAK_BF16,
+              2.0 * (S * ctx * dk + T * H * (dk + rank)), f"{T} rows x {H} heads x ~{int(keys)} keys of {dk}+{rank}, bf16 MFMA peak")
+        # the Mixtral-shaped model's attention: 128-wide heads, 4 query heads per kv head
+        G = max(width // 512, 1)
+        kv = rnd(S * nb, 1, 2, G, bs, 128)
+        q3 = rnd(T, H, 128)
+        if mode == "prefill":
+            fn = lambda: ops.paged_attention_prefill(q3, kv[:, 0], bt, qsl, seq, 0.09, T)  # noqa: E731
+        else:
+            fn = lambda: ops.paged_attention_decode(q3, kv[:, 0], bt, seq, 0.09, ctx)  # noqa: E731
+        t = _time(fn, 5)
+        entry(f"paged_attention/{mode} (mixtral)", t, 2.0 * T * H * keys * 256, PEAK_BF16,
+              2.0 * (S * ctx * G * 256 + 2 * T * H * 128), f"{T} rows x {H} heads x ~{int(keys)} keys of 128+128, bf16 MFMA peak")
+        fr = rotary_frequencies(dr, 10000.0, None).to(dev)
+        dqv, dkvv = rnd(T, qr), rnd(T, dk)
+        qn, kn = torch.ones(qr, device=dev).to(dt), torch.ones(rank, device=dev).to(dt)
+        t = _time(lambda: seqmix.latent_prep(dqv, dkvv, pos, slots, cache, 0, rank, bs, fr, qn, kn, 1e-5), 5)
+        entry(f"latent_prep/{mode}", t, 0.0, PEAK_F32, 4.0 * T * (qr + dk), f"{T} rows: both latents read, normed / turned, written")
+        qh = rnd(T, H * 192)
+        t = _time(lambda: seqmix.rope_half_into(q, qh, pos, H, 192, 128, dk, rank, fr), 5)
+        entry(f"rope_half_into/{mode}", t, 0.0, PEAK_F32, 4.0 * T * H * dr, f"{T} rows x {H} heads x {dr} turned entries")
+        # routed experts: router, the two expert products with the capped activation, the sum
+        f = RoutedExperts("f.", width, E, top, ff, 7.0)
+        w = {"f.router": rnd(E, width), "f._gu": rnd(E, 2 * ff, width) * width ** -0.5, "f._down": rnd(E, width, ff) * ff ** -0.5}
+        h = rnd(T, width)
+        t = _time(lambda: f.forward(h, w), 5)
+        act = min(E, T * top)
+        entry(f"routed_experts/{mode}", t, 6.0 * T * top * width * ff, PEAK_BF16, 2.0 * (3 * act * width * ff + 2 * T * width),
+              f"{T} rows x {top} of {E} experts of {ff}, bf16 MFMA peak; {act} experts' weights read once")
+        w13 = rnd(E, 2 * ff, width) * width ** -0.5
+        w2 = rnd(E, width, ff) * ff ** -0.5
+        gate = rnd(E, width)
+
+        def mixtral_moe():
+            tw, ti = ops.moe_topk_softmax(ops.linear(h, gate), top)
+            return moe_ops.fused_experts(h, w13, w2, tw, ti, 0)
+        t = _time(mixtral_moe, 5)
+        entry(f"routed_experts/{mode} (mixtral)", t, 6.0 * T * top * width * ff, PEAK_BF16,
+              2.0 * (3 * act * width * ff + 2 * T * width), f"{T} rows x {top} of {E} experts of {ff}, bf16 MFMA peak")
+        gu = rnd(T * top, 2 * ff)
+        t = _time(lambda: seqmix.capped_glu(gu, 7.0), 5)
+        entry(f"capped_glu/{mode}", t, 0.0, PEAK_F32, 6.0 * T * top * ff, f"{T * top} rows x {ff}: gate and up in, product out")
+        t = _time(lambda: seqmix.silu_mul(gu), 5)
+        entry(f"silu_mul/{mode} (tapasun)", t, 0.0, PEAK_F32, 6.0 * T * top * ff, f"{T * top} rows x {ff}: gate and up in, product out")
+    return out
+
+
 def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4, only: str = "all",
          design: str = "voletar") -> int:
-    """only: all | tapasun | voletar | llama | kernels (e.g. one model alone under a profiler)."""
+    """only: all | momuvik | mixtral | tapasun | voletar | llama | kernels (e.g. one model alone under a profiler)."""
     from .. import ops
     ops.ext()
     for width in sizes:
@@ -276,8 +386,11 @@ def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4, on
             if only in ("all", name.split("-")[0]):
                 print(json.dumps(run_model(name, prompt, batch, context)), flush=True)
         if only in ("all", "kernels"):
-            rows = (tapasun_rooflines(width, prompt, batch, context) if design == "tapasun" else []) + \
-                kernel_rooflines(width, prompt, batch, context)
+            if design == "momuvik":
+                rows = momuvik_rooflines(width, prompt, batch, context)
+            else:
+                rows = (tapasun_rooflines(width, prompt, batch, context) if design == "tapasun" else []) + \
+                    kernel_rooflines(width, prompt, batch, context)
             for e in rows:
                 print(json.dumps(e), flush=True)
     return 0
