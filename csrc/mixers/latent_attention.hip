@@ -44,17 +44,21 @@ __device__ __forceinline__ s4_t hi4(const uint4& a) {
 constexpr int kPartHead = 4;  // floats ahead of a stretch's output: maximum, sum, two unused (16-byte rows)
 
 // KKM: 32-entry chunks of a row (dk <= 32 KKM); VTM: 16-entry value tiles (rank <= 16 VTM); NW: waves of
-// a workgroup (its LDS is NW transposed value blocks)
-template <int KKM, int VTM, int NW>
+// a workgroup (its LDS is NW transposed value blocks); QLDS: the query pieces wait in LDS, each lane's
+// own 16 bytes per chunk side by side, instead of in registers (the widest rows: the output
+// accumulator and a block's key pieces already take 200 registers)
+// EXACT: dk = 32 KKM and rank = 16 VTM, so no piece or tile needs a bounds test
+template <int KKM, int VTM, int NW, bool QLDS, bool EXACT>
 __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ cache, long block_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ qsl, const int* __restrict__ seq_lens, int koff, int H, int dk, int rank, float scale,
     const float* __restrict__ sink, int nsplit) {
-  extern __shared__ __attribute__((aligned(16))) bf16_t vt_lds[];  // [NW waves][16 VTM entries][kVtPitch]
+  extern __shared__ __attribute__((aligned(16))) bf16_t vt_lds[];  // [NW waves][16 VTM entries][kVtPitch] (+ [NW][KKM][64] x 16 B)
   const int s = blockIdx.z;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   bf16_t* vt_w = vt_lds + wid * (16 * VTM * kVtPitch);
+  uint4* q_l = reinterpret_cast<uint4*>(vt_lds + NW * (16 * VTM * kVtPitch)) + wid * (KKM * 64) + lane;
   const int row0 = qsl[s], qlen = qsl[s + 1] - row0;
   const int nrows = qlen * H;
   const int id = blockIdx.x * NW + wid;
@@ -74,15 +78,18 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
   const int nblk = (p_last >> 4) + 1;
   const int b0 = static_cast<int>(static_cast<long>(nblk) * sp / nsplit);
   const int b1 = static_cast<int>(static_cast<long>(nblk) * (sp + 1) / nsplit);
-  const int KK = (dk + 31) >> 5, VT = rank >> 4;
+  const int KK = EXACT ? KKM : (dk + 31) >> 5, VT = EXACT ? VTM : rank >> 4;
   const int* bt = block_tables + static_cast<long>(s) * bt_stride;
-  uint4 qf[KKM];
+  uint4 qf[QLDS ? 1 : KKM];
   {
     const bf16_t* qp = q + static_cast<long>(row0 + tok) * q_stride + static_cast<long>(hd) * dk + 8 * kg;
 #pragma unroll
-    for (int kk = 0; kk < KKM; ++kk)
-      qf[kk] = (kk < KK && rok && 32 * kk + 8 * kg + 8 <= dk) ? *reinterpret_cast<const uint4*>(qp + 32 * kk)
-                                                              : make_uint4(0, 0, 0, 0);
+    for (int kk = 0; kk < KKM; ++kk) {
+      const uint4 v = (rok && (EXACT || (kk < KK && 32 * kk + 8 * kg + 8 <= dk))) ? *reinterpret_cast<const uint4*>(qp + 32 * kk)
+                                                                                  : make_uint4(0, 0, 0, 0);
+      if (QLDS) q_l[kk * 64] = v;  // read back by this lane only
+      else qf[kk] = v;
+    }
   }
   const float L2E = 1.4426950408889634f;
   float m = (sink && sp == 0) ? sink[hd] * L2E : -INFINITY;
@@ -96,30 +103,34 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
     const bf16_t* kp = cache + static_cast<long>(bt[kb]) * block_stride + koff + static_cast<long>(c) * dk + 8 * kg;
 #pragma unroll
     for (int kk = 0; kk < KKM; ++kk)
-      kr[kk] = (kk < KK && 32 * kk + 8 * kg + 8 <= dk) ? *reinterpret_cast<const uint4*>(kp + 32 * kk)
-                                                       : make_uint4(0, 0, 0, 0);
+      kr[kk] = (EXACT || (kk < KK && 32 * kk + 8 * kg + 8 <= dk)) ? *reinterpret_cast<const uint4*>(kp + 32 * kk)
+                                                                  : make_uint4(0, 0, 0, 0);
+    // key rows past the tile's last position may hold anything (also NaN); no row of the tile sees
+    // them, but as values they would be multiplied by their zero weights: read them as zeros.  Only a
+    // tile's last block can have such rows.
+    if (kb * 16 + 15 > p_last && kb * 16 + c > p_last) {
+#pragma unroll
+      for (int kk = 0; kk < KKM; ++kk) kr[kk] = make_uint4(0, 0, 0, 0);
+    }
   };
   if (b0 < b1) load_block(b0);
   for (int kb = b0; kb < b1; ++kb) {
     const int k0 = kb * 16;
-    f4_t acc = f4_t{0.f, 0.f, 0.f, 0.f};
+    __builtin_amdgcn_wave_barrier();  // the previous block's LDS reads come before this block's writes
+    // four accumulators: consecutive MFMAs do not wait for one another
+    f4_t ac[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ac[i] = f4_t{0.f, 0.f, 0.f, 0.f};
+    // the block's values go into the wave's LDS area transposed, piece by piece as the scores are summed
 #pragma unroll
     for (int kk = 0; kk < KKM; ++kk) {
-      if (kk < KK) {
-        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(lo4(kr[kk]), lo4(qf[kk]), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(hi4(kr[kk]), hi4(qf[kk]), acc, 0, 0, 0);
-      }
-    }
-    // the block's values, transposed, into the wave's LDS area; rows past the tile's last position
-    // may hold anything (also NaN): they are written as zeros
-    __builtin_amdgcn_wave_barrier();  // the previous block's reads come first
-    {
-      const bool kok = k0 + c <= p_last;
-#pragma unroll
-      for (int kk = 0; kk < KKM; ++kk) {
+      if (EXACT || kk < KK) {
+        const uint4 qv = QLDS ? q_l[kk * 64] : qf[QLDS ? 0 : kk];
+        ac[(2 * kk) & 3] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(lo4(kr[kk]), lo4(qv), ac[(2 * kk) & 3], 0, 0, 0);
+        ac[(2 * kk + 1) & 3] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(hi4(kr[kk]), hi4(qv), ac[(2 * kk + 1) & 3], 0, 0, 0);
         const int d0 = 32 * kk + 8 * kg;
-        if (kk < KK && d0 < rank) {
-          const uint4 a = kok ? kr[kk] : make_uint4(0, 0, 0, 0);
+        if (d0 < rank) {
+          const uint4 a = kr[kk];
           bf16_t* w = vt_w + d0 * kVtPitch + c;
           w[0] = static_cast<bf16_t>(a.x & 0xFFFFu);
           w[kVtPitch] = static_cast<bf16_t>(a.x >> 16);
@@ -132,6 +143,7 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
         }
       }
     }
+    const f4_t acc = (ac[0] + ac[1]) + (ac[2] + ac[3]);
     if (kb + 1 < b1) load_block(kb + 1);  // in flight while the weights are made and the values multiplied
     // a block that every row of the tile sees whole needs no mask
     const bool whole = k0 + 15 <= p_first;
@@ -175,7 +187,7 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
     const bf16_t* vp = vt_w + c * kVtPitch + 4 * kg;
 #pragma unroll
     for (int vt = 0; vt < VTM; ++vt) {
-      if (vt < VT) {
+      if (EXACT || vt < VT) {
         const s4_t a = *reinterpret_cast<const s4_t*>(vp + 16 * vt * kVtPitch);
         const f4_t t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, o[vt], 0, 0, 0);
         o[vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, t, 0, 0, 0);
@@ -207,28 +219,36 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
   }
 }
 
-// One workgroup per (token, head) row: the stretches' (m, l, o) merged.  m is in log2 units.
+// One workgroup per (token, head) row: the stretches' (m, l, o) merged.  m is in log2 units.  The
+// stretches' weights 2^(m_s - M) / L are made once by the first wave's lanes; the sum over the
+// stretches is unrolled so that their loads are in flight together.
+constexpr int kMaxSplit = 64;
 __global__ void __launch_bounds__(128) latent_attention_combine_kernel(bf16_t* __restrict__ out,
                                                                        const float* __restrict__ part, int nsplit,
                                                                        int rank) {
+  __shared__ float wsh[kMaxSplit];
   const long row = blockIdx.x;
   const int ps = rank + kPartHead;
   const float* pp = part + row * nsplit * ps;
-  float M = -INFINITY;
-  for (int s = 0; s < nsplit; ++s) M = fmaxf(M, pp[s * ps]);
-  float L = 0.f;
-  for (int s = 0; s < nsplit; ++s) {
-    const float ms = pp[s * ps];
-    if (ms != -INFINITY) L += pp[s * ps + 1] * __builtin_amdgcn_exp2f(ms - M);
+  if (threadIdx.x < 64) {
+    const int s = threadIdx.x;
+    const float ms = s < nsplit ? pp[s * ps] : -INFINITY;
+    const float ls = s < nsplit ? pp[s * ps + 1] : 0.f;
+    const float M = wave_max(ms);
+    const float w = ms != -INFINITY ? __builtin_amdgcn_exp2f(ms - M) : 0.f;
+    const float L = wave_sum(ls * w);
+    wsh[s] = w / L;
   }
-  const float inv = 1.f / L;
+  __syncthreads();
   for (int d = threadIdx.x; d < rank; d += blockDim.x) {
+    const float* pd = pp + kPartHead + d;
     float a = 0.f;
+#pragma unroll 8
     for (int s = 0; s < nsplit; ++s) {
-      const float ms = pp[s * ps];
-      if (ms != -INFINITY) a += pp[s * ps + kPartHead + d] * __builtin_amdgcn_exp2f(ms - M);
+      const float w = wsh[s];
+      a += w != 0.f ? pd[s * ps] * w : 0.f;  // a stretch without keys wrote zeros; nothing is read as a number it is not
     }
-    out[row * rank + d] = f2bf(a * inv);
+    out[row * rank + d] = f2bf(a);
   }
 }
 
@@ -240,17 +260,18 @@ bool launch_latent_attention(void* out, float* part, const void* q, long q_strid
   if (rows == 0 || S == 0) return true;
   if (bs != 16 || dk % 8 || rank % 16 || rank > dk || dk > 576 || rank > 512 || q_stride % 8 || koff % 8 ||
       block_stride % 8 || reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(cache) % 16 ||
-      reinterpret_cast<uintptr_t>(part) % 16 || nsplit < 1 || (nsplit > 1 && part == nullptr))
+      reinterpret_cast<uintptr_t>(part) % 16 || nsplit < 1 || nsplit > kMaxSplit || (nsplit > 1 && part == nullptr))
     return false;
   const int tiles = (max_q * H + 15) / 16;
-#define MIX_LA(KKM, VTM, NW)                                                                                          \
-  hipLaunchKernelGGL((latent_attention_mfma_kernel<KKM, VTM, NW>), dim3((tiles * nsplit + NW - 1) / NW, 1, S),        \
-                     dim3(64 * NW), NW * 16 * VTM * kVtPitch * sizeof(bf16_t), st, (bf16_t*)out, part,                \
-                     (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride, qsl,    \
-                     seq_lens, koff, H, dk, rank, scale, sink, nsplit)
-  if (dk <= 192 && rank <= 128) MIX_LA(6, 8, 4);
-  else if (dk <= 320 && rank <= 256) MIX_LA(10, 16, 4);
-  else MIX_LA(18, 32, 2);  // 40 KB of LDS for two waves
+#define MIX_LA(KKM, VTM, NW, QLDS, EXACT)                                                                             \
+  hipLaunchKernelGGL((latent_attention_mfma_kernel<KKM, VTM, NW, QLDS, EXACT>), dim3((tiles * nsplit + NW - 1) / NW, 1, S), \
+                     dim3(64 * NW), NW * (16 * VTM * kVtPitch * sizeof(bf16_t) + (QLDS ? KKM * 64 * 16 : 0)), st,     \
+                     (bf16_t*)out, part, (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, \
+                     bt_stride, qsl, seq_lens, koff, H, dk, rank, scale, sink, nsplit)
+  if (dk <= 192 && rank <= 128) MIX_LA(6, 8, 4, false, false);
+  else if (dk <= 320 && rank <= 256) MIX_LA(10, 16, 4, false, false);
+  else if (dk == 576 && rank == 512) MIX_LA(18, 32, 1, true, true);
+  else MIX_LA(18, 32, 1, true, false);  // 38 KB of LDS a wave: four one-wave workgroups share a CU
 #undef MIX_LA
   MXS_CHECK_LAUNCH();
   if (nsplit > 1) {

@@ -9,7 +9,7 @@ tensors, re-pack them once when the weights are loaded, and compute from a step'
                  scores weigh each expert's INPUT (optionally renormalised); an optional shared
                  CappedExpert with its own size and limit sees every token unweighted
 
-The kernels are in mxserve/ops/seqmix.py (csrc/mixers/experts.hip on the GPU); the matrix products go
+The kernels are in mxserve/ops/seqmix.py (csrc/mixers/latent_experts.hip on the GPU); the matrix products go
 through ops.linear and torch.bmm (hipBLASLt).
 """
 from __future__ import annotations
@@ -83,7 +83,8 @@ class RoutedExperts(FeedForward):
                 got rows (one host read of the E + 1 offsets), expert_combine gathers each token's rows
     """
 
-    BATCHED_MAX_TOKENS = 32
+    BATCHED_MAX_TOKENS = 32    # always batched up to this many tokens ...
+    BATCHED_MAX_ROWS = 1024    # ... and beyond while experts x tokens stays within this many rows
 
     def __init__(self, prefix: str, width: int, experts: int, top: int, ff: int, limit: float,
                  shared: Optional[CappedExpert] = None, alpha: float = 1.702, renorm: bool = False):
@@ -118,7 +119,7 @@ class RoutedExperts(FeedForward):
         extra = self.shared.forward(h, w) if self.shared is not None else None
         gu, down = w[p + "_gu"], w[p + "_down"]
         capturing = h.is_cuda and torch.cuda.is_current_stream_capturing()
-        if T <= self.BATCHED_MAX_TOKENS or capturing:
+        if T <= self.BATCHED_MAX_TOKENS or T * self.E <= self.BATCHED_MAX_ROWS or capturing:
             xs = seqmix.spread_scaled(h, tw, ids, self.E)  # [E, T, W]
             a = seqmix.capped_glu(torch.bmm(xs, gu.transpose(1, 2)).view(self.E * T, -1), self.limit, self.alpha)
             ys = torch.bmm(a.view(self.E, T, -1), down.transpose(1, 2))  # [E, T, W]
