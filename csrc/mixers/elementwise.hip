@@ -108,13 +108,25 @@ __global__ void __launch_bounds__(256) gated_rms_norm_kernel(T* __restrict__ out
 template <typename T>
 __global__ void __launch_bounds__(256) gate_linear_kernel(float* __restrict__ out, const T* __restrict__ h, long h_stride,
                                                           const T* __restrict__ w, const T* __restrict__ bias, int N,
-                                                          int W) {
+                                                          int W, int vec) {
+  constexpr int EL = El<T>::N;
   const long row = blockIdx.x;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const T* hr = h + row * h_stride;
   for (int n = wid; n < N; n += nw) {
     float s = 0.f;
-    for (int c = lane; c < W; c += 64) s += ldf(hr + c) * ldf(w + static_cast<long>(n) * W + c);
+    const T* wr = w + static_cast<long>(n) * W;
+    if (vec) {  // rows of whole, aligned 16-byte pieces
+      for (int c = lane * EL; c < W; c += 64 * EL) {
+        float a[EL], b[EL];
+        load16(hr + c, a);
+        load16(wr + c, b);
+#pragma unroll
+        for (int e = 0; e < EL; ++e) s += a[e] * b[e];
+      }
+    } else {
+      for (int c = lane; c < W; c += 64) s += ldf(hr + c) * ldf(wr + c);
+    }
     s = wave_sum(s);
     if (lane == 0) out[row * N + n] = s + (bias ? ldf(bias + n) : 0.f);
   }
@@ -189,8 +201,11 @@ void launch_gated_rms_norm(void* out, const float* o, const void* gate, long g_s
 void launch_gate_linear(float* out, const void* h, long h_stride, const void* w, const void* bias, int rows, int N,
                         int W, bool bf, hipStream_t st) {
   if (rows == 0) return;
+  const int el = bf ? 8 : 4;
+  const int vec = W % el == 0 && h_stride % el == 0 && reinterpret_cast<uintptr_t>(h) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(w) % 16 == 0;
   MIX_DISPATCH(bf, hipLaunchKernelGGL(gate_linear_kernel<T>, dim3(rows), dim3(256), 0, st, out, (const T*)h, h_stride,
-                                      (const T*)w, (const T*)bias, N, W));
+                                      (const T*)w, (const T*)bias, N, W, vec));
   MXS_CHECK_LAUNCH();
 }
 

@@ -176,8 +176,31 @@ __global__ void __launch_bounds__(256) spread_scaled_kernel(T* __restrict__ xs, 
 template <typename T>
 __global__ void __launch_bounds__(256) expert_combine_kernel(T* __restrict__ out, const T* __restrict__ ys,
                                                              const int* __restrict__ index, int k, long row_stride,
-                                                             const T* __restrict__ extra, long extra_stride, int W) {
+                                                             const T* __restrict__ extra, long extra_stride, int W,
+                                                             int vec) {
+  constexpr int EL = El<T>::N;
   const long t = blockIdx.x;
+  if (vec) {  // rows of whole, aligned 16-byte pieces: the k rows' loads of a piece are in flight together
+    for (int c = threadIdx.x * EL; c < W; c += blockDim.x * EL) {
+      float s[EL];
+      if (extra) {
+        load16(extra + t * extra_stride + c, s);
+      } else {
+#pragma unroll
+        for (int e = 0; e < EL; ++e) s[e] = 0.f;
+      }
+#pragma unroll 4
+      for (int j = 0; j < k; ++j) {
+        const long r = index ? index[t * k + j] : j * row_stride + t;
+        float v[EL];
+        load16(ys + r * W + c, v);
+#pragma unroll
+        for (int e = 0; e < EL; ++e) s[e] += v[e];
+      }
+      store16(out + t * W + c, s);
+    }
+    return;
+  }
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float s = extra ? ldf(extra + t * extra_stride + c) : 0.f;
     for (int j = 0; j < k; ++j) {
@@ -252,8 +275,11 @@ void launch_spread_scaled(void* xs, const void* h, long h_stride, const float* w
 void launch_expert_combine(void* out, const void* ys, const int* index, int Tn, int k, long row_stride, const void* extra,
                            long extra_stride, int W, bool bf, hipStream_t st) {
   if (Tn == 0) return;
+  const int el = bf ? 8 : 4;
+  const int vec = W % el == 0 && extra_stride % el == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
+                  reinterpret_cast<uintptr_t>(ys) % 16 == 0 && reinterpret_cast<uintptr_t>(extra) % 16 == 0;
   MIX_DISPATCH(bf, hipLaunchKernelGGL(expert_combine_kernel<T>, dim3(Tn), dim3(256), 0, st, (T*)out, (const T*)ys, index, k,
-                                      row_stride, (const T*)extra, extra_stride, W));
+                                      row_stride, (const T*)extra, extra_stride, W, vec));
   MXS_CHECK_LAUNCH();
 }
 

@@ -40,6 +40,28 @@ template <> __device__ __forceinline__ float dot_row<bf16_t>(const float* __rest
   return s;
 }
 
+// 16 bytes of a row as floats: 8 bf16 or 4 fp32 (the pointer is 16-byte aligned)
+template <typename T> struct El;
+template <> struct El<bf16_t> { static constexpr int N = 8; };
+template <> struct El<float> { static constexpr int N = 4; };
+__device__ __forceinline__ void load16(const bf16_t* p, float* o) {
+  const uint4 a = *reinterpret_cast<const uint4*>(p);
+  o[0] = bf2f_lo(a.x); o[1] = bf2f_hi(a.x); o[2] = bf2f_lo(a.y); o[3] = bf2f_hi(a.y);
+  o[4] = bf2f_lo(a.z); o[5] = bf2f_hi(a.z); o[6] = bf2f_lo(a.w); o[7] = bf2f_hi(a.w);
+}
+__device__ __forceinline__ void load16(const float* p, float* o) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+__device__ __forceinline__ void store16(bf16_t* p, const float* v) {
+  uint4 a;
+  a.x = pack2(v[0], v[1]); a.y = pack2(v[2], v[3]); a.z = pack2(v[4], v[5]); a.w = pack2(v[6], v[7]);
+  *reinterpret_cast<uint4*>(p) = a;
+}
+__device__ __forceinline__ void store16(float* p, const float* v) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+}
+
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
 __device__ __forceinline__ float logsigmoid_f(float z) { return z < 0.f ? z - log1pf(expf(z)) : -log1pf(expf(-z)); }

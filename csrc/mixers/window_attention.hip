@@ -94,19 +94,6 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
 // scattered 16-byte) pieces; the score is summed over the eight lanes.  The value rows are read the
 // same way with the weight of their key, and the 32 key slots of the block are summed at the end
 // (three lane exchanges, then the four waves through LDS).
-template <typename T> struct El;
-template <> struct El<bf16_t> { static constexpr int N = 8; };
-template <> struct El<float> { static constexpr int N = 4; };
-__device__ __forceinline__ void load16(const bf16_t* p, float* o) {
-  const uint4 a = *reinterpret_cast<const uint4*>(p);
-  o[0] = bf2f_lo(a.x); o[1] = bf2f_hi(a.x); o[2] = bf2f_lo(a.y); o[3] = bf2f_hi(a.y);
-  o[4] = bf2f_lo(a.z); o[5] = bf2f_hi(a.z); o[6] = bf2f_lo(a.w); o[7] = bf2f_hi(a.w);
-}
-__device__ __forceinline__ void load16(const float* p, float* o) {
-  const float4 a = *reinterpret_cast<const float4*>(p);
-  o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
-}
-
 // NC: 128-byte stretches of a row (head sizes <= NC * 8 * El<T>::N).  RM: query heads of one kv head that
 // a workgroup serves together: a key or value row is loaded once and used for all of them.
 template <typename T, int NC, int RM>
