@@ -36,7 +36,7 @@ void launch_gated_norm(void*, long, const float*, const void*, long, const void*
                        float, bool, hipStream_t);
 bool launch_column_scan(const ScanArgs&, int, bool, bool, hipStream_t);
 bool launch_latent_attention(void*, float*, const void*, long, const void*, long, const int*, int, const int*, const int*,
-                             int, int, int, int, int, int, int, float, int, const float*, int, hipStream_t);
+                             int, int, int, int, int, int, int, float, int, const float*, int, bool, hipStream_t);
 void launch_latent_prep(void*, const void*, long, const void*, long, const int64_t*, const int64_t*, void*, long, int, int,
                         int, int, int, int, const float*, const void*, const void*, float, bool, hipStream_t);
 void launch_rope_half_into(void*, long, const void*, long, const int64_t*, int, int, int, int, int, int, const float*, int,
@@ -462,7 +462,7 @@ void latent_prep(at::Tensor cq, at::Tensor dq, at::Tensor dkv, at::Tensor positi
 // was launched and the caller runs window_attention with strided value rows instead.
 bool latent_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor block_tables, at::Tensor qsl,
                       at::Tensor seq_lens, int64_t koff, int64_t H, int64_t dk, int64_t rank, int64_t bs, double scale,
-                      int64_t max_query_len, OptT sink, int64_t nsplit, OptT part) {
+                      int64_t max_query_len, OptT sink, int64_t nsplit, OptT part, bool pair) {
   if (!is_bf(q)) return false;
   const float* sinkp = nullptr;
   if (sink.has_value()) {
@@ -486,7 +486,7 @@ bool latent_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor
       block_tables.data_ptr<int>(), static_cast<int>(block_tables.stride(0)), i32(qsl, S + 1, "qsl"),
       i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(koff), static_cast<int>(H),
       static_cast<int>(dk), static_cast<int>(rank), static_cast<int>(bs), static_cast<float>(scale),
-      static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(max_query_len, T))), sinkp, static_cast<int>(nsplit), stream());
+      static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(max_query_len, T))), sinkp, static_cast<int>(nsplit), pair, stream());
 }
 
 void rope_half_into(at::Tensor out, at::Tensor x, at::Tensor positions, int64_t heads, int64_t x_dim, int64_t x_col,

@@ -5,12 +5,11 @@
 // The rows of a sequence's step are its (token, head) pairs, flattened; a wave owns 16 consecutive
 // rows and walks the 16-key cache blocks that its rows see (causal), or one of `nsplit` stretches of
 // them.  No workgroup barriers: the four waves of a workgroup are independent.  Per block, with
-// v_mfma_f32_16x16x16_bf16:
+// v_mfma_f32_16x16x32_bf16 (scores) and v_mfma_f32_16x16x16_bf16 (values):
 //   S^T = K Q^T      A = the block's 16 key rows, loaded from the pages as 16-byte pieces that are
 //                    used as they are: lane (key c, group kg) holds entries 32 kk + 8 kg .. + 7 of its
-//                    key, the two halves of a piece feed two MFMAs, and Q^T (held in registers for
-//                    the whole walk) is loaded in the same order, so the products pair up whatever
-//                    the order of the summed index is.  The accumulator has the row on the lane
+//                    key, one piece feeds one 32-deep MFMA, and Q^T (held in registers for
+//                    the whole walk) is loaded in the same order, so the products pair up.  The accumulator has the row on the lane
 //                    and 4 keys per lane: maxima and sums are per-lane work plus two lane exchanges.
 //   O^T += V^T P^T   B = P^T straight from the S^T accumulator's registers, every weight split into
 //                    two bf16 halves (p = hi + lo, two MFMAs) so that the product keeps 16 mantissa
@@ -27,19 +26,13 @@ namespace mxs {
 
 typedef short s4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef __bf16 bf8_t __attribute__((ext_vector_type(8)));
+// one v_mfma_f32_16x16x32_bf16 per 16-byte piece: lane (c, kg) holds the 8 summed indices 8 kg .. 8 kg + 7
+__device__ __forceinline__ f4_t mfma_piece(const uint4& a, const uint4& b, f4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf8_t, a), __builtin_bit_cast(bf8_t, b), c, 0, 0, 0);
+}
 
 constexpr int kVtPitch = 20;  // bf16 per transposed row: 16 keys + 4, so that the four key groups fall into different banks
-
-__device__ __forceinline__ s4_t lo4(const uint4& a) {
-  union { uint2 u; s4_t s; } x;
-  x.u = make_uint2(a.x, a.y);
-  return x.s;
-}
-__device__ __forceinline__ s4_t hi4(const uint4& a) {
-  union { uint2 u; s4_t s; } x;
-  x.u = make_uint2(a.z, a.w);
-  return x.s;
-}
 
 constexpr int kPartHead = 4;  // floats ahead of a stretch's output: maximum, sum, two unused (16-byte rows)
 
@@ -126,8 +119,7 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
     for (int kk = 0; kk < KKM; ++kk) {
       if (EXACT || kk < KK) {
         const uint4 qv = QLDS ? q_l[kk * 64] : qf[QLDS ? 0 : kk];
-        ac[(2 * kk) & 3] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(lo4(kr[kk]), lo4(qv), ac[(2 * kk) & 3], 0, 0, 0);
-        ac[(2 * kk + 1) & 3] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(hi4(kr[kk]), hi4(qv), ac[(2 * kk + 1) & 3], 0, 0, 0);
+        ac[kk & 3] = mfma_piece(kr[kk], qv, ac[kk & 3]);
         const int d0 = 32 * kk + 8 * kg;
         if (d0 < rank) {
           const uint4 a = kr[kk];
@@ -219,6 +211,180 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
   }
 }
 
+// ---- Pair form for the widest rows: a workgroup of two waves owns one 16-row tile and splits the ROW
+// between them.  Wave w multiplies its half of the 32-entry chunks (half of the score products; the two
+// partial score tiles meet in LDS and both waves add them in the same order, so both hold the same
+// weights), writes its chunks' share of the transposed values into the workgroup's LDS block, and
+// accumulates its half of the value tiles.  A wave then holds 64 accumulators, 36 registers of query
+// pieces and 36 of key pieces: two such waves fit a SIMD, and one covers the other's waits.  Two
+// workgroup barriers per key block (of two waves each): before the transposed values are overwritten, and
+// after they and the partial scores are written.  24 KB of LDS a workgroup: four share a CU.
+template <int KKM, int VTM, bool EXACT>
+__global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))) latent_attention_pair_kernel(
+    bf16_t* __restrict__ out, float* __restrict__ part, const bf16_t* __restrict__ q, long q_stride,
+    const bf16_t* __restrict__ cache, long block_stride, const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ qsl, const int* __restrict__ seq_lens, int koff, int H, int dk, int rank, float scale,
+    const float* __restrict__ sink, int nsplit) {
+  constexpr int KHM = KKM / 2, VHM = VTM / 2;
+  static_assert(KKM % 2 == 0 && VTM % 2 == 0, "the row is split in two");
+  __shared__ __attribute__((aligned(16))) bf16_t vt_s[16 * VTM * kVtPitch];
+  __shared__ __attribute__((aligned(16))) f4_t sx[2][2][64];
+  const int s = blockIdx.z;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int row0 = qsl[s], qlen = qsl[s + 1] - row0;
+  const int nrows = qlen * H;
+  const int id = blockIdx.x;
+  const int tile = id / nsplit, sp = id - tile * nsplit;
+  if (tile * 16 >= nrows) return;  // the same for both waves of the workgroup
+  const int c = lane & 15, kg = lane >> 4;
+  const int r = tile * 16 + c;
+  const bool rok = r < nrows;
+  const int rr = rok ? r : nrows - 1;
+  const int tok = rr / H, hd = rr - tok * H;
+  const int last = bt_stride * 16 - 1;
+  const int base = max(seq_lens[s] - qlen, 0);
+  const int pq = min(base + tok, last);
+  const int p_first = min(base + (tile * 16) / H, last);
+  const int p_last = min(base + min(tile * 16 + 15, nrows - 1) / H, last);
+  const int nblk = (p_last >> 4) + 1;
+  const int b0 = static_cast<int>(static_cast<long>(nblk) * sp / nsplit);
+  const int b1 = static_cast<int>(static_cast<long>(nblk) * (sp + 1) / nsplit);
+  const int KK = EXACT ? KKM : (dk + 31) >> 5, VT = EXACT ? VTM : rank >> 4;
+  const int kk0 = w * KHM, vt0 = w * VHM;  // this wave's chunks and value tiles
+  const int* bt = block_tables + static_cast<long>(s) * bt_stride;
+  uint4 qf[KHM];
+  {
+    const bf16_t* qp = q + static_cast<long>(row0 + tok) * q_stride + static_cast<long>(hd) * dk + 8 * kg;
+#pragma unroll
+    for (int j = 0; j < KHM; ++j) {
+      const int kk = kk0 + j;
+      qf[j] = (rok && (EXACT || (kk < KK && 32 * kk + 8 * kg + 8 <= dk))) ? *reinterpret_cast<const uint4*>(qp + 32 * kk)
+                                                                          : make_uint4(0, 0, 0, 0);
+    }
+  }
+  const float L2E = 1.4426950408889634f;
+  float m = (sink && sp == 0) ? sink[hd] * L2E : -INFINITY;
+  float l = (sink && sp == 0 && kg == 0) ? 1.f : 0.f;
+  f4_t o[VHM];
+#pragma unroll
+  for (int j = 0; j < VHM; ++j) o[j] = f4_t{0.f, 0.f, 0.f, 0.f};
+  const float sl2 = scale * L2E;
+  uint4 kr[KHM];
+  auto load_block = [&](int kb) {
+    const bf16_t* kp = cache + static_cast<long>(bt[kb]) * block_stride + koff + static_cast<long>(c) * dk + 8 * kg;
+#pragma unroll
+    for (int j = 0; j < KHM; ++j) {
+      const int kk = kk0 + j;
+      kr[j] = (EXACT || (kk < KK && 32 * kk + 8 * kg + 8 <= dk)) ? *reinterpret_cast<const uint4*>(kp + 32 * kk)
+                                                                 : make_uint4(0, 0, 0, 0);
+    }
+    if (kb * 16 + 15 > p_last && kb * 16 + c > p_last) {  // stale rows behind the tile's last position: zeros
+#pragma unroll
+      for (int j = 0; j < KHM; ++j) kr[j] = make_uint4(0, 0, 0, 0);
+    }
+  };
+  if (b0 < b1) load_block(b0);
+  for (int kb = b0; kb < b1; ++kb) {
+    const int k0 = kb * 16, buf = (kb - b0) & 1;
+    bf16_t* vt_w = vt_s;
+    __syncthreads();  // both waves have read the previous block's values
+    f4_t ac[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) ac[i] = f4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int j = 0; j < KHM; ++j) {
+      const int kk = kk0 + j;
+      if (EXACT || kk < KK) {
+        ac[j & 3] = mfma_piece(kr[j], qf[j], ac[j & 3]);
+        const int d0 = 32 * kk + 8 * kg;
+        if (d0 < rank) {
+          const uint4 a = kr[j];
+          bf16_t* wp = vt_w + d0 * kVtPitch + c;
+          wp[0] = static_cast<bf16_t>(a.x & 0xFFFFu);
+          wp[kVtPitch] = static_cast<bf16_t>(a.x >> 16);
+          wp[2 * kVtPitch] = static_cast<bf16_t>(a.y & 0xFFFFu);
+          wp[3 * kVtPitch] = static_cast<bf16_t>(a.y >> 16);
+          wp[4 * kVtPitch] = static_cast<bf16_t>(a.z & 0xFFFFu);
+          wp[5 * kVtPitch] = static_cast<bf16_t>(a.z >> 16);
+          wp[6 * kVtPitch] = static_cast<bf16_t>(a.w & 0xFFFFu);
+          wp[7 * kVtPitch] = static_cast<bf16_t>(a.w >> 16);
+        }
+      }
+    }
+    sx[buf][w][lane] = (ac[0] + ac[1]) + (ac[2] + ac[3]);
+    if (kb + 1 < b1) load_block(kb + 1);  // in flight across the barrier, the weights and the value products
+    __syncthreads();
+    const f4_t acc = sx[buf][0][lane] + sx[buf][1][lane];  // the same sum in both waves
+    const bool whole = k0 + 15 <= p_first;
+    float sv[4], mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (whole) {
+        sv[i] = acc[i] * sl2;
+      } else {
+        const int jj = k0 + 4 * kg + i;
+        sv[i] = (rok && jj <= pq) ? acc[i] * sl2 : -INFINITY;
+      }
+      mx = fmaxf(mx, sv[i]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {
+      const float corr = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m - m_new);
+      l *= corr;
+#pragma unroll
+      for (int j = 0; j < VHM; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[j][i] *= corr;
+      m = m_new;
+    }
+    s4_t ph, pl;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float pr = (whole || sv[i] != -INFINITY) ? __builtin_amdgcn_exp2f(sv[i] - m) : 0.f;
+      l += pr;
+      const uint32_t u = __float_as_uint(pr), uh = u & 0xFFFF0000u;
+      uint32_t ul = __float_as_uint(pr - __uint_as_float(uh));
+      ul += 0x7FFFu + ((ul >> 16) & 1u);
+      ph[i] = static_cast<short>(uh >> 16);
+      pl[i] = static_cast<short>(ul >> 16);
+    }
+    const bf16_t* vp = vt_w + (16 * vt0 + c) * kVtPitch + 4 * kg;
+#pragma unroll
+    for (int j = 0; j < VHM; ++j) {
+      if (EXACT || vt0 + j < VT) {
+        const s4_t a = *reinterpret_cast<const s4_t*>(vp + 16 * j * kVtPitch);
+        const f4_t t = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, o[j], 0, 0, 0);
+        o[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, t, 0, 0, 0);
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!rok) return;
+  const long grow = static_cast<long>(row0 + tok) * H + hd;
+  if (nsplit == 1) {
+    const float inv = 1.f / l;
+    bf16_t* op = out + grow * rank + 16 * vt0 + 4 * kg;
+#pragma unroll
+    for (int j = 0; j < VHM; ++j) {
+      if (EXACT || vt0 + j < VT) {
+        uint2 wv;
+        wv.x = pack2(o[j][0] * inv, o[j][1] * inv);
+        wv.y = pack2(o[j][2] * inv, o[j][3] * inv);
+        *reinterpret_cast<uint2*>(op + 16 * j) = wv;
+      }
+    }
+  } else {
+    float* pp = part + (grow * nsplit + sp) * (rank + kPartHead);
+    if (kg == 0 && w == 0) { pp[0] = m; pp[1] = l; }
+#pragma unroll
+    for (int j = 0; j < VHM; ++j)
+      if (EXACT || vt0 + j < VT) *reinterpret_cast<f4_t*>(pp + kPartHead + 16 * (vt0 + j) + 4 * kg) = o[j];
+  }
+}
+
 // One workgroup per (token, head) row: the stretches' (m, l, o) merged.  m is in log2 units.  The
 // stretches' weights 2^(m_s - M) / L are made once by the first wave's lanes; the sum over the
 // stretches is unrolled so that their loads are in flight together.
@@ -256,7 +422,7 @@ __global__ void __launch_bounds__(128) latent_attention_combine_kernel(bf16_t* _
 bool launch_latent_attention(void* out, float* part, const void* q, long q_stride, const void* cache, long block_stride,
                              const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S, int rows,
                              int koff, int H, int dk, int rank, int bs, float scale, int max_q, const float* sink,
-                             int nsplit, hipStream_t st) {
+                             int nsplit, bool pair, hipStream_t st) {
   if (rows == 0 || S == 0) return true;
   if (bs != 16 || dk % 8 || rank % 16 || rank > dk || dk > 576 || rank > 512 || q_stride % 8 || koff % 8 ||
       block_stride % 8 || reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(cache) % 16 ||
@@ -270,6 +436,15 @@ bool launch_latent_attention(void* out, float* part, const void* q, long q_strid
                      bt_stride, qsl, seq_lens, koff, H, dk, rank, scale, sink, nsplit)
   if (dk <= 192 && rank <= 128) MIX_LA(6, 8, 4, false, false);
   else if (dk <= 320 && rank <= 256) MIX_LA(10, 16, 4, false, false);
+  else if (pair) {
+#define MIX_LP(EXACT)                                                                                                  \
+  hipLaunchKernelGGL((latent_attention_pair_kernel<18, 32, EXACT>), dim3(tiles * nsplit, 1, S), dim3(128), 0, st,      \
+                     (bf16_t*)out, part, (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, \
+                     bt_stride, qsl, seq_lens, koff, H, dk, rank, scale, sink, nsplit)
+    if (dk == 576 && rank == 512) MIX_LP(true);
+    else MIX_LP(false);
+#undef MIX_LP
+  }
   else if (dk == 576 && rank == 512) MIX_LA(18, 32, 1, true, true);
   else MIX_LA(18, 32, 1, true, false);  // 38 KB of LDS a wave: four one-wave workgroups share a CU
 #undef MIX_LA

@@ -633,6 +633,9 @@ def rope_half_into(out: torch.Tensor, x: torch.Tensor, positions: torch.Tensor, 
 
 
 LATENT_TARGET_WAVES = 1024  # waves that fill the 256 CUs one deep: single-token steps split their keys up to this
+# the widest rows (over 320 entries): "pair" = two waves per 16-row tile, each half of the row; "single" = one wave
+# per tile with its queries in LDS; "auto" = pair
+LATENT_WIDE_FORM = os.environ.get("MXS_LATENT_WIDE_FORM", "auto")
 
 
 def latent_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, qsl: torch.Tensor,
@@ -656,7 +659,8 @@ def latent_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
         part = (torch.empty(T * num_heads * nsplit * (rank + 4), dtype=torch.float32, device=q.device)
                 if nsplit > 1 else None)
         if ext().latent_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), num_heads, dk, rank, block_size,
-                                  float(scale), mq, sink, nsplit, part):
+                                  float(scale), mq, sink, nsplit, part,
+                                  LATENT_WIDE_FORM != "single"):
             return out
     return window_attention(q, cache, block_tables, qsl, seq_lens, koff, koff, num_heads, 1, dk, rank, block_size, scale,
                             0, 0, max_query_len, sink=sink, v_stride=dk)

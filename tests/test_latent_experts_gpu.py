@@ -35,10 +35,11 @@ def _case(H, dk, rank, lens, qlens, seed=0, sink=True, stale=float("nan")):
     return q, cache, bt, qsl, torch.tensor(lens, dtype=torch.int32), sk
 
 
-@pytest.mark.parametrize("H,dk,rank", [(8, 160, 128), (3, 48, 32), (16, 576, 512), (12, 320, 256), (5, 136, 112), (40, 64, 64)])
+@pytest.mark.parametrize("H,dk,rank", [(8, 160, 128), (3, 48, 32), (16, 576, 512), (12, 320, 256), (5, 136, 112), (40, 64, 64),
+                                       (6, 408, 352), (2, 552, 512)])
 @pytest.mark.parametrize("lens,qlens", [([300], [300]), ([77, 130, 16, 250], [1, 1, 1, 1]), ([100, 45, 333], [1, 45, 21]),
                                          ([17], [2])])
-def test_latent_attention_kernel(H, dk, rank, lens, qlens):
+def test_latent_attention_kernel(H, dk, rank, lens, qlens, monkeypatch):
     if not torch.cuda.is_available():
         pytest.skip("no GPU")
     q, cache, bt, qsl, sl, sk = _case(H, dk, rank, lens, qlens, seed=H + dk)
@@ -48,10 +49,12 @@ def test_latent_attention_kernel(H, dk, rank, lens, qlens):
     dev = torch.device("cuda")
     cg = cache.to(torch.bfloat16).to(dev)  # with the stale rows as they are
     args = (qb.to(dev), cg, bt.to(dev), qsl.to(dev), sl.to(dev), 8, H, dk, rank, 16, 0.11)
-    for max_seq in (max(lens), 16):  # keys split over several waves where the step is small, and never
-        got = seqmix.latent_attention(*args, max(qlens), max_seq, sink=None if sk is None else sk.to(dev))
-        err = (got.float().cpu() - want).abs().max().item()
-        assert err < 0.02, f"max abs error {err}"
+    for form in ("single", "pair"):  # the two forms of the widest size class (the others have one)
+        monkeypatch.setattr(seqmix, "LATENT_WIDE_FORM", form)
+        for max_seq in (max(lens), 16):  # keys split over several waves where the step is small, and never
+            got = seqmix.latent_attention(*args, max(qlens), max_seq, sink=None if sk is None else sk.to(dev))
+            err = (got.float().cpu() - want).abs().max().item()
+            assert err < 0.02, f"{form}: max abs error {err}"
     # the general kernel on the same operands (strided value rows)
     got = seqmix.window_attention(args[0], cg, args[2], args[3], args[4], 8, 8, H, 1, dk, rank, 16, 0.11, 0, 0, max(qlens),
                                   sink=None if sk is None else sk.to(dev), v_stride=dk)
