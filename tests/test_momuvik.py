@@ -34,15 +34,21 @@ def _row_errors(got, want):
 
 def _check(got, want, tol, margins=None):
     """fp32 (tol well below 1e-2): every row within tol.  bf16: the mean over the rows (of eight or
-    more) within tol / 4 and the worst row within 2.5 tol, where a row whose routing was a close call
-    in the oracle is left out: rounding may send it to another expert."""
+    more) within tol / 4 and the worst row within 2.5 tol -- up to the sequence's first token whose
+    routing was a close call in the oracle: rounding may send that token to another expert, and every
+    later token attends to what it left in the pages.  From there on the rows must stay near (median
+    within tol, none beyond 1): a mechanism that fails does not."""
     if tol < 1e-2:
         e = rel_err(got, want)
         assert e < tol, f"relative error {e:.3g} >= {tol}"
         return
     e = _row_errors(got, want)
-    if margins is not None:
-        e = e[np.asarray(margins) >= CLOSE]
+    assert np.isfinite(e).all()
+    if margins is not None and (np.asarray(margins) < CLOSE).any():
+        first = int(np.argmax(np.asarray(margins) < CLOSE))
+        after = e[first:]
+        assert np.median(after) < tol and after.max() < 1.0, f"rows after a close call: median {np.median(after):.3g}, worst {after.max():.3g}"
+        e = e[:first]
     assert (len(e) < 8 or e.mean() < tol / 4) and (len(e) == 0 or e.max() < 2.5 * tol), \
         f"row errors: mean {e.mean():.3g}, worst {e.max():.3g} (tol {tol})"
 
