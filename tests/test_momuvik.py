@@ -461,24 +461,28 @@ VARIANTS = {
     "equal_sizes_everywhere": config([layer(latent(heads=2, dim=16, rot_dim=16, vdim=16, kv_rank=16, q_rank=16), dense(16)),
                                       layer(latent(heads=2, dim=16, rot_dim=16, vdim=16, kv_rank=16, q_rank=16),
                                             moe(experts=16, top=16, ff=16, limit=1.0, shared=(16, 1.0)))], width=16, vocab=16),
+    "sizes_that_fit_no_vector_load": config([layer(latent(heads=3, dim=10, rot_dim=6, vdim=7, kv_rank=12, q_rank=9, scale=0.3),
+                                                   moe(experts=3, top=2, ff=14, limit=1.1, shared=(5, 0.9))),
+                                             layer(latent(heads=5, dim=6, rot_dim=2, vdim=9, kv_rank=21, q_rank=11, scale=0.4), dense(22))],
+                                            width=50, vocab=37),
     "wide_latent_many_heads": config([layer(latent(heads=12, dim=8, rot_dim=40, vdim=72, kv_rank=264, q_rank=136, scale=0.07),
                                             moe(experts=9, top=4, ff=40, limit=1.5, shared=(72, 0.5)))], width=72, vocab=60),
 }
 
 
-@pytest.mark.parametrize("dev", DEVS)
+@pytest.mark.parametrize("dev,dtype,tol", DEV_DTYPE_TOL)
 @pytest.mark.parametrize("name", list(VARIANTS))
-def test_other_sizes(tmp_path, dev, name):
+def test_other_sizes(tmp_path, dev, dtype, tol, name):
     _skip(dev)
     cfg = VARIANTS[name]
     w = write_checkpoint(tmp_path, cfg, seed=5)
     t = _tokens(45, cfg["vocab"], 6)
-    want, _ = _oracle_model(cfg, w, t)
-    eng = engine(tmp_path, dev, "float32", max_tokens=128)
+    want, margins = _oracle_model(cfg, w, t)
+    eng = engine(tmp_path, dev, dtype, max_tokens=128)
     for sizes in ([1000], [20, 2, 1, 7, 1]):
         steps = [[("a", p, False)] for p in cut(t, sizes)]
         steps[-1] = [("a", steps[-1][0][1], True)]
-        _check(replay(eng, steps)["a"], want, 1e-4)
+        _check(replay(eng, steps)["a"], want, tol, margins)
 
 
 @pytest.mark.parametrize("dev", DEVS)
