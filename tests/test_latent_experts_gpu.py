@@ -35,7 +35,7 @@ def _case(H, dk, rank, lens, qlens, seed=0, sink=True, stale=float("nan")):
     return q, cache, bt, qsl, torch.tensor(lens, dtype=torch.int32), sk
 
 
-@pytest.mark.parametrize("H,dk,rank", [(8, 160, 128), (3, 48, 32), (16, 576, 512), (12, 320, 256), (5, 136, 112), (40, 64, 64),
+@pytest.mark.parametrize("H,dk,rank", [(10, 184, 96), (3, 48, 32), (16, 576, 512), (12, 320, 256), (5, 136, 112), (40, 64, 64),
                                        (6, 408, 352), (2, 552, 512)])
 @pytest.mark.parametrize("lens,qlens", [([300], [300]), ([77, 130, 16, 250], [1, 1, 1, 1]), ([100, 45, 333], [1, 45, 21]),
                                          ([17], [2])])
