@@ -18,7 +18,7 @@ from typing import Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str  # "llama" | "qwen3" | "mixtral" | "voletar" | "tapasun" | "momuvik"
+    arch: str  # "llama" | "qwen3" | "mixtral" | "voletar" | "tapasun" | "momuvik" | "seradra"
     hidden_size: int
     intermediate_size: int
     num_layers: int
@@ -40,7 +40,7 @@ class ModelConfig:
     bos_token_id: Optional[int] = None
     eos_token_ids: list = field(default_factory=list)
     chat_template: str = "llama3"
-    # designs whose config lists their layers (arch "voletar", "tapasun", "momuvik"): the checkpoint's own
+    # designs whose config lists their layers (arch "voletar", "tapasun", "momuvik", "seradra"): the checkpoint's own
     # config.json structure -- per-layer mixer type and sizes, norm eps and the design's other
     # constants -- as the design's module (mxserve/models/<arch>.py) reads it.  None for the uniform
     # transformer families.
@@ -287,7 +287,55 @@ _reg(momuvik_config("tiny-momuvik", {
         {"type": "latent_attention", "mixer": _latent(2, 32, 8, 32, 24, 32, 0.15), "mlp": None}]}))
 
 
+def seradra_config(name: str, d: dict) -> ModelConfig:
+    """A Seradra checkpoint's config.json: `width`, `vocab`, `norm.eps`, `layers` (each with `type` attention |
+    latent_attention, `mixer`, `mlp` dense | moe | null).  The uniform fields are filled from the first layer
+    for the code that sizes things from them."""
+    layers = d["layers"]
+    att = layers[0]["mixer"] if layers else {"heads": 1, "dim": int(d["width"])}
+    latent = bool(layers) and layers[0]["type"] == "latent_attention"
+    ffs = [int(l["mlp"]["ff"]) if l["mlp"].get("kind", "dense") == "dense" else int(l["mlp"]["expert"]["ff"])
+           for l in layers if l.get("mlp")]
+    moes = [l["mlp"]["router"] for l in layers if l.get("mlp") and l["mlp"].get("kind") == "moe"]
+    keep = {k: d[k] for k in ("layers", "norm", "width", "vocab") if k in d}
+    return ModelConfig(
+        name=name, arch="seradra", hidden_size=int(d["width"]), intermediate_size=max(ffs) if ffs else 0,
+        num_layers=len(layers), num_heads=int(att["heads"]),
+        num_kv_heads=1 if latent else int(att.get("kv_heads", att["heads"])),
+        head_dim=int(att["dim"]) + (int(att["rot_dim"]) if latent else 0), vocab_size=int(d["vocab"]),
+        rms_norm_eps=float((d.get("norm") or {}).get("eps", 1e-5)), tie_word_embeddings=False,
+        max_position_embeddings=int(d.get("max_position_embeddings", 1 << 20)),
+        num_experts=max((int(r["experts"]) for r in moes), default=0),
+        num_experts_per_tok=max((int(r["top"]) for r in moes), default=0),
+        bos_token_id=d.get("bos_token_id"), eos_token_ids=list(d.get("eos_token_ids") or []),
+        chat_template="chatml", arch_config=keep)
+
+
+def _talking(heads, kv_heads, dim, vdim, scale, window, rot_dims, base=10000.0, scaling=None):
+    rot = {"dims": rot_dims, "base": base}
+    if scaling:
+        rot["scaling"] = scaling
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale, "mask": {"size": window},
+            "rot": rot}
+
+
+# A small Seradra (random weights): both mixers, a dense and a routed feed-forward, a layer without one.
+_reg(seradra_config("tiny-seradra", {
+    "architecture": "Seradra", "width": 96, "vocab": 384, "norm": {"eps": 1e-5},
+    "layers": [
+        {"type": "attention", "mlp": {"kind": "dense", "ff": 160},
+         "mixer": _talking(4, 2, 32, 16, 0.2, 24, 16, 10000.0,
+                           {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 1.0})},
+        {"type": "latent_attention", "mlp": {"kind": "moe", "router": {"experts": 6, "top": 2}, "expert": {"ff": 48}},
+         "mixer": dict(_latent(3, 24, 16, 16, 48, 24, 0.16, 5000.0), mask={"size": 20})},
+        {"type": "attention", "mlp": None, "mixer": _talking(3, 3, 16, 32, 0.25, 40, 8, 3000.0)},
+        {"type": "latent_attention", "mlp": {"kind": "dense", "ff": 128},
+         "mixer": dict(_latent(4, 16, 8, 24, 32, 40, 0.2), mask={"size": 33})}]}))
+
+
 def _from_hf_json(name: str, d: dict) -> ModelConfig:
+    if d.get("architecture") == "Seradra":
+        return seradra_config(name, d)
     if d.get("architecture") == "Momuvik":
         return momuvik_config(name, d)
     if d.get("architecture") == "Voletar":

@@ -1,5 +1,5 @@
 """What the designs whose config lists their layers share (mxserve/models/voletar.py,
-mxserve/models/tapasun.py, mxserve/models/momuvik.py): the plan of layer runs with every run's place inside a cache block and a
+mxserve/models/tapasun.py, mxserve/models/momuvik.py, mxserve/models/seradra.py): the plan of layer runs with every run's place inside a cache block and a
 state slot, and the model surface the runner expects (weights in a flat dict, the mixers' input
 projections fused into one GEMM per layer, cache geometry from the plan).
 
@@ -18,7 +18,7 @@ from ..parallel.comm import get_tp
 from .config import ModelConfig
 from .mixers import Mixer
 
-HYBRID_ARCHS = ("voletar", "tapasun", "momuvik")
+HYBRID_ARCHS = ("voletar", "tapasun", "momuvik", "seradra")
 
 
 def design_module(arch: str):

@@ -525,4 +525,7 @@ def build_model(cfg: ModelConfig, device, dtype=torch.bfloat16, moe_dispatch: st
     if cfg.arch == "momuvik":
         from .momuvik import MomuvikLM
         return MomuvikLM(cfg, device, dtype, block_size)
+    if cfg.arch == "seradra":
+        from .seradra import SeradraLM
+        return SeradraLM(cfg, device, dtype, block_size)
     return TransformerLM(cfg, device, dtype, moe_dispatch)

@@ -24,9 +24,13 @@ in a slot) and computes its output from a step's flattened token batch.
                         output projection over their concatenated activations
   LatentAttention       softmax attention whose keys and values are expansions of one normed low-rank
                         latent per token plus one rotated key part shared by the heads (half-split
-                        rotary pairs), queries through a normed latent of their own, optional learned
-                        sink; only the latent and the rotated part are cached, the expansions are
-                        folded into the query and the output
+                        or neighbouring rotary pairs), queries through a normed latent of their own,
+                        optional learned sink, optional sliding window; only the latent and the rotated
+                        part are cached, the expansions are folded into the query and the output
+  TalkingAttention      softmax attention whose heads' scores are mixed by a learned [H, H] matrix before
+                        the softmax; projections with biases, one RMS norm over all query rows and one
+                        over all key rows, half-split rotary pairs on part of each head with
+                        ramp-blended frequencies and a factor on cos / sin, sliding window, learned sink
 
 The kernels are in mxserve/ops/seqmix.py (csrc/mixers/*.hip on the GPU).
 """
@@ -196,11 +200,28 @@ def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None) -
     """fp32 [dims / 2]: base^(-2i/dims), computed in float64 on the host.  scaling {factor}: every
     frequency divided by factor.  scaling {factor, low, high, original}: by wavelength l = 2 pi / f,
     kept where l < original / high, divided by factor where l > original / low, and in between blended
-    with s = (original / l - low) / (high - low) as (1 - s) f / factor + s f."""
+    with s = (original / l - low) / (high - low) as (1 - s) f / factor + s f.
+    scaling {factor, original, fast, slow}: a ramp over the pair index i between the indices at which
+    `fast` and `slow` turns fit into `original` positions, x(t) = dims ln(original / (2 pi t)) / (2 ln base):
+    lo = max(floor(x(fast)), 0), hi = min(ceil(x(slow)), dims - 1), r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),
+    frequency r_i f / factor + (1 - r_i) f (rotary_magnitude() gives the factor on cos and sin that goes with it)."""
     f = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
     if scaling:
         factor = float(scaling["factor"])
-        if "original" in scaling:
+        if "fast" in scaling:
+            orig = float(scaling["original"])
+
+            def index_of(turns: float) -> float:
+                return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+            lo = max(math.floor(index_of(float(scaling["fast"]))), 0)
+            hi = min(math.ceil(index_of(float(scaling["slow"]))), dims - 1)
+            out = []
+            for i, fi in enumerate(f):
+                r = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+                out.append(fi / factor * r + fi * (1.0 - r))
+            f = out
+        elif "original" in scaling:
             orig, low, high = float(scaling["original"]), float(scaling["low"]), float(scaling["high"])
             out = []
             for fi in f:
@@ -216,6 +237,13 @@ def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None) -
         else:
             f = [fi / factor for fi in f]
     return torch.tensor(f, dtype=torch.float64).to(torch.float32)
+
+
+def rotary_magnitude(scaling: Optional[dict]) -> float:
+    """The factor on cos and sin that goes with ramp-blended frequencies: 0.1 ln(factor) + 1."""
+    if scaling and "fast" in scaling:
+        return 0.1 * math.log(float(scaling["factor"])) + 1.0
+    return 1.0
 
 
 def _fp32(w: dict, name: str) -> None:
@@ -470,14 +498,20 @@ class LatentAttention(Mixer):
     row's first kv_rank entries, so nothing is stored twice.  W_uk is folded into the query
     (q'_h = [W_uk,h^T q_h,plain | q_h,rot], score = scale * q'_h . [c | r]) and W_uv is applied to the
     weighted sum of latents: every head attends over the same rows, with head sizes kv_rank + rot_dim
-    and kv_rank.  sink: None | "learned" (tensor `<prefix>sink` [heads])."""
+    and kv_rank.  sink: None | "learned" (tensor `<prefix>sink` [heads]).  window > 0: position i sees the
+    positions i - window + 1 .. i.  split_pairs: coordinate i of the rotated part pairs with i + rot_dim / 2
+    (False: 2i with 2i + 1)."""
 
     def __init__(self, prefix: str, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
-                 q_rank: int, scale: float, rot: dict, sink: Optional[str] = "learned"):
+                 q_rank: int, scale: float, rot: dict, sink: Optional[str] = "learned", window: int = 0,
+                 split_pairs: bool = True):
         if int(rot["dims"]) != rot_dim or rot_dim % 2:
             raise ValueError(f"{prefix}: the rotated part has rot_dim = rot.dims entries, an even number")
         if sink not in (None, "learned"):
             raise ValueError(f"{prefix}: unknown sink {sink!r}")
+        if window < 0:
+            raise ValueError(f"{prefix}: window {window}")
+        self.window, self.split_pairs = int(window), bool(split_pairs)
         self.p, self.width = prefix, width
         self.heads, self.dn, self.dr, self.vd = int(heads), int(dim), int(rot_dim), int(vdim)
         self.rank, self.q_rank, self.scale, self.sink = int(kv_rank), int(q_rank), float(scale), sink
@@ -509,19 +543,82 @@ class LatentAttention(Mixer):
         dq, dkv = parts
         T = h.shape[0]
         cq = seqmix.latent_prep(dq, dkv, md.positions, md.slot_mapping, ctx.cache, koff, self.rank, ctx.block_size,
-                                self.freqs, w[p + "dq.norm"], w[p + "dkv.norm"], ctx.eps)
+                                self.freqs, w[p + "dq.norm"], w[p + "dkv.norm"], ctx.eps, self.split_pairs)
         q = ops.linear(cq, w[p + "uq"])  # [T, H * (dn + dr)]
         dq_, dk = self.dn + self.dr, self.dk
         qf = torch.empty(T, H * dk, dtype=q.dtype, device=q.device)
         # the plain part through W_uk^T, head by head, straight into its columns of the folded query
         torch.bmm(q.view(T, H, dq_)[:, :, :self.dn].transpose(0, 1), w[p + "uk"],
                   out=qf.view(T, H, dk)[:, :, :self.rank].transpose(0, 1))
-        seqmix.rope_half_into(qf, q, md.positions, H, dq_, self.dn, dk, self.rank, self.freqs)
+        seqmix.rope_half_into(qf, q, md.positions, H, dq_, self.dn, dk, self.rank, self.freqs, self.split_pairs)
         lat = seqmix.latent_attention(qf, ctx.cache, md.block_tables, md.query_start_loc, md.seq_lens, koff, H, dk,
                                       self.rank, ctx.block_size, self.scale, md.max_query_len,
-                                      getattr(md, "max_seq_len", 0), sink=w.get(p + "sink"))
+                                      getattr(md, "max_seq_len", 0), sink=w.get(p + "sink"), window=self.window)
         o = torch.empty(T, H * self.vd, dtype=q.dtype, device=q.device)
         torch.bmm(lat.view(T, H, self.rank).transpose(0, 1), w[p + "uv"], out=o.view(T, H, self.vd).transpose(0, 1))
+        return ops.linear(o, w[p + "o"])
+
+
+class TalkingAttention(Mixer):
+    """q = W_q h + b_q, k, v likewise; q and k each RMS-normed over ALL their rows at once (weights
+    `<prefix>q.norm` [H dk], `<prefix>k.norm` [G dk]); the first rot.dims coordinates of every head turned as
+    pairs (i, i + rot.dims / 2); score_h = sum_g talk[h, g] scale q_g . k_g (`<prefix>talk` [H, H], mixed
+    before the mask and the softmax); window > 0: position i sees i - window + 1 .. i; sink: None | "learned"
+    (`<prefix>sink` [H], one more term exp(sink_h) in the denominator).  bias / whole_norm / talk can each
+    be switched off for a design that lacks them."""
+
+    def __init__(self, prefix: str, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, rot: dict,
+                 window: int = 0, sink: Optional[str] = "learned", bias: bool = True, whole_norm: bool = True,
+                 talk: bool = True):
+        if heads % kv_heads:
+            raise ValueError(f"{prefix}: {heads} query heads do not divide over {kv_heads} kv heads")
+        rd = int(rot["dims"])
+        if rd % 2 or rd > dim:
+            raise ValueError(f"{prefix}: rotary pairs need an even number of dimensions inside the head")
+        if sink not in (None, "learned") or window < 0:
+            raise ValueError(f"{prefix}: sink {sink!r}, window {window}")
+        self.p, self.width = prefix, width
+        self.heads, self.kv_heads, self.dk, self.dv = heads, kv_heads, dim, vdim
+        self.scale, self.window, self.sink = float(scale), int(window), sink
+        self.bias, self.whole_norm, self.talk = bool(bias), bool(whole_norm), bool(talk)
+        sc = rot.get("scaling") or None
+        self.freqs = rotary_frequencies(rd, float(rot["base"]), sc)
+        self.mag = rotary_magnitude(sc)
+
+    def proj_rows(self) -> list:
+        return [(self.p + "q", self.heads * self.dk), (self.p + "k", self.kv_heads * self.dk),
+                (self.p + "v", self.kv_heads * self.dv)]
+
+    def extra_shapes(self) -> dict:
+        p, H, G = self.p, self.heads, self.kv_heads
+        sh = {p + "o": (self.width, H * self.dv)}
+        if self.bias:
+            sh.update({p + "q.b": (H * self.dk,), p + "k.b": (G * self.dk,), p + "v.b": (G * self.dv,)})
+        if self.whole_norm:
+            sh.update({p + "q.norm": (H * self.dk,), p + "k.norm": (G * self.dk,)})
+        if self.talk:
+            sh[p + "talk"] = (H, H)
+        if self.sink == "learned":
+            sh[p + "sink"] = (H,)
+        return sh
+
+    def finish_weights(self, w: dict) -> None:
+        self.freqs = self.freqs.to(w[self.p + "o"].device)
+        if self.talk:
+            _fp32(w, self.p + "talk")
+        if self.sink == "learned":
+            _fp32(w, self.p + "sink")
+
+    def forward(self, parts: list, h: torch.Tensor, w: dict, ctx: StepContext, koff: int, voff: int, soff: int):
+        q, k, v = parts
+        md, p = ctx.md, self.p
+        seqmix.rope_qkv_cache(q, k, v, md.positions, md.slot_mapping, ctx.cache, koff, voff, self.heads, self.kv_heads,
+                              self.dk, self.dv, ctx.block_size, self.freqs, w.get(p + "q.norm"), w.get(p + "k.norm"),
+                              ctx.eps, bias_q=w.get(p + "q.b"), bias_k=w.get(p + "k.b"), bias_v=w.get(p + "v.b"),
+                              norm_whole=self.whole_norm, split_pairs=True, mag=self.mag)
+        o = seqmix.window_attention(q, ctx.cache, md.block_tables, md.query_start_loc, md.seq_lens, koff, voff,
+                                    self.heads, self.kv_heads, self.dk, self.dv, ctx.block_size, self.scale, self.window,
+                                    0, md.max_query_len, sink=w.get(p + "sink"), talk=w.get(p + "talk"))
         return ops.linear(o, w[p + "o"])
 
 

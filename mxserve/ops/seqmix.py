@@ -65,25 +65,30 @@ def resid_update(x: torch.Tensor, a: Optional[torch.Tensor], eps: float, *, wa: 
                  b: Optional[torch.Tensor] = None, wb: Optional[torch.Tensor] = None,
                  bias: Optional[torch.Tensor] = None, assign: bool = False,
                  norm_w: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None,
-                 a_scale: float = 1.0, w_offset: float = 0.0):
+                 a_scale: float = 1.0, w_offset: float = 0.0, wa_offset: float = 0.0,
+                 cast_dtype: Optional[torch.dtype] = None):
     """One pass over the fp32 residual stream x [T, W], in place:
-        d = a * a_scale            (wa: RMSNorm(a) * wa)
+        d = a * a_scale            (wa: RMSNorm(a) * (wa_offset + wa))
         d = (d + RMSNorm(b) * wb) / 2      when b is given (two branches, each normed over the width)
         d += bias                  (a [W] vector)
         x = d if assign else x + d
     and, when norm_w is given, returns RMSNorm(x) * (w_offset + norm_w) in out_dtype (the next
     sublayer's input; w_offset = 1 for weights stored as their difference from one, added in fp32).
-    a = None leaves x as it is (norm only).  All sums and norms in fp32."""
+    Without norm_w, cast_dtype asks for the updated x itself in that dtype (a next sublayer that
+    reads the stream un-normed).  a = None leaves x as it is.  All sums and norms in fp32."""
     if _gpu(x):
         h = None
         if norm_w is not None:
             h = torch.empty(x.shape, dtype=out_dtype or norm_w.dtype, device=x.device)
-        ext().resid_update(x, a, wa, b, wb, bias, bool(assign), norm_w, h, float(eps), float(a_scale), float(w_offset))
+        elif cast_dtype is not None:
+            h = torch.empty(x.shape, dtype=cast_dtype, device=x.device)
+        ext().resid_update(x, a, wa, b, wb, bias, bool(assign), norm_w, h, float(eps), float(a_scale), float(w_offset),
+                           float(wa_offset))
         return h
     if a is not None:
         d = a.float() * a_scale if a_scale != 1.0 else a.float()
         if wa is not None:
-            d = _rms(d, eps) * wa.float()
+            d = _rms(d, eps) * (wa.float() + wa_offset if wa_offset else wa.float())
         if b is not None:
             d = 0.5 * (d + _rms(b.float(), eps) * wb.float())
         if bias is not None:
@@ -93,8 +98,37 @@ def resid_update(x: torch.Tensor, a: Optional[torch.Tensor], eps: float, *, wa: 
         else:
             x.add_(d)
     if norm_w is None:
-        return None
+        return None if cast_dtype is None else x.to(cast_dtype, copy=True)
     return (_rms(x, eps) * (norm_w.float() + w_offset if w_offset else norm_w.float())).to(out_dtype or norm_w.dtype)
+
+
+def embed_normed(ids: torch.Tensor, table: torch.Tensor, w: torch.Tensor, eps: float, w_offset: float,
+                 out: torch.Tensor, cast_dtype: Optional[torch.dtype] = None):
+    """out (fp32 [T, W], may be one slab of a larger buffer) = RMSNorm(table[ids]) * (w_offset + w): an
+    embedding that is normed before it becomes the stream.  Returns out in cast_dtype when asked."""
+    if _gpu(table):
+        h = torch.empty(out.shape, dtype=cast_dtype, device=out.device) if cast_dtype is not None else None
+        ext().embed_normed(out, h, ids, table, w, float(eps), float(w_offset))
+        return h
+    out.copy_(_rms(F.embedding(ids, table).float(), eps) * (w.float() + w_offset))
+    return None if cast_dtype is None else out.to(cast_dtype, copy=True)
+
+
+def depth_mix(hist: torch.Tensor, n: int, coeffs: torch.Tensor, cast_dtype: Optional[torch.dtype] = None):
+    """hist fp32 [L, T, W]: slab n <- sum over j < n of coeffs[j] * slab j (coeffs fp32 [n]): a stream
+    that goes on as a weighted sum of everything earlier layers produced.  Returns the new slab in
+    cast_dtype when asked.  fp32 products and sums, in the order of j."""
+    if not 0 < n < hist.shape[0] or coeffs.numel() != n:
+        raise ValueError(f"depth_mix: slab {n} of {hist.shape[0]} with {coeffs.numel()} coefficients")
+    if _gpu(hist):
+        h = torch.empty(hist.shape[1:], dtype=cast_dtype, device=hist.device) if cast_dtype is not None else None
+        ext().depth_mix(hist, int(n), coeffs, h)
+        return h
+    acc = hist[0] * coeffs[0]
+    for j in range(1, n):
+        acc = acc + hist[j] * coeffs[j]
+    hist[n].copy_(acc)
+    return None if cast_dtype is None else hist[n].to(cast_dtype, copy=True)
 
 
 def cast_into(dst: torch.Tensor, x: torch.Tensor) -> None:
@@ -112,6 +146,18 @@ def relu_sq(x: torch.Tensor) -> torch.Tensor:
         ext().relu_sq(out, x)
         return out
     return F.relu(x.float()).square().to(x.dtype)
+
+
+def xielu(x: torch.Tensor, ab: torch.Tensor) -> torch.Tensor:
+    """ab fp32 [2] = (a, b), both positive:  z > 0: a z^2 + z / 2;  z <= 0: b (e^z - 1 - z) + z / 2.
+    Computed in fp32."""
+    if _gpu(x):
+        out = torch.empty_like(x)
+        ext().xielu(out, x, ab)
+        return out
+    z = x.float()
+    zn = z.clamp(max=0.0)
+    return torch.where(z > 0, ab[0] * z * z + 0.5 * z, ab[1] * (torch.expm1(zn) - zn) + 0.5 * z).to(x.dtype)
 
 
 def softcap(x: torch.Tensor, cap: float) -> torch.Tensor:
@@ -167,7 +213,8 @@ def kv_write(cache: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_mapping
 def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, qsl: torch.Tensor,
                      seq_lens: torch.Tensor, koff: int, voff: int, num_heads: int, num_kv_heads: int, dk: int,
                      dv: int, block_size: int, scale: float, window: int, keep_first: int,
-                     max_query_len: int = 0, sink: Optional[torch.Tensor] = None, v_stride: int = 0) -> torch.Tensor:
+                     max_query_len: int = 0, sink: Optional[torch.Tensor] = None, v_stride: int = 0,
+                     talk: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Softmax attention over the paged cache (this step's keys already written).  The query at
     position i sees key j <= i when i - j < window or j < keep_first (window <= 0: every j <= i).
     q [T, H*dk] (row-strided view) -> [T, H*dv] in q's dtype; scores and weights in fp32.
@@ -175,8 +222,19 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
     holds exp(sink[h]), a key without a value whose score is not scaled.  v_stride (elements, 0: dv): the
     distance between two tokens' value rows, for values that are a slice of a wider cached row (then
     num_kv_heads is 1 and voff points at the slice inside the first row).  max_query_len: the longest chunk of the step (host
-    int); from 16 rows a bf16 step with head sizes that are multiples of 16 runs the MFMA kernel."""
+    int); from 16 rows a bf16 step with head sizes that are multiples of 16 runs the MFMA kernel.
+    talk (fp32 [H, H]): the heads' scaled scores of a (query, key) pair are mixed before the softmax,
+    score_h <- sum_g talk[h, g] score_g (the mask and the sink act on the mixed scores); a workgroup then
+    serves all heads of its rows."""
     T = q.shape[0]
+    if _gpu(q) and talk is not None:
+        if v_stride and v_stride != dv:
+            raise ValueError("mixed heads read value rows back to back")
+        out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
+        ext().talking_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), int(voff), num_heads, num_kv_heads,
+                                dk, dv, block_size, float(scale), int(window), int(keep_first), int(max_query_len), sink,
+                                talk)
+        return out
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
         ext().window_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), int(voff), num_heads,
@@ -205,6 +263,8 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
         V = vc[blocks].permute(0, 2, 1, 3).reshape(nb * block_size, num_kv_heads, dv)[:n].float()
         qs = q[a:e].reshape(e - a, num_heads, dk).float()
         sc = torch.einsum("mhd,nhd->hmn", qs, K.repeat_interleave(g, dim=1)) * scale
+        if talk is not None:
+            sc = torch.einsum("hg,gmn->hmn", talk.float(), sc)
         i = torch.arange(n - (e - a), n).unsqueeze(1)
         j = torch.arange(n).unsqueeze(0)
         seen = j <= i
@@ -352,11 +412,11 @@ def silu_mul(gu: torch.Tensor) -> torch.Tensor:
 
 
 # ----------------------------------------------------------------------------- rotary positions
-def _rotate(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor, sign: float) -> torch.Tensor:
+def _rotate(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor, sign: float, mag: float = 1.0) -> torch.Tensor:
     """x fp32 [T, heads, dim]: pair (2i, 2i+1) turned by sign * pos * freqs[i]; the rest passes."""
     n = freqs.numel()
     ang = pos.to(torch.float32).view(-1, 1, 1) * freqs.float().view(1, 1, n) * sign
-    c, s = torch.cos(ang), torch.sin(ang)
+    c, s = torch.cos(ang) * mag, torch.sin(ang) * mag
     u, v = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
     y = x.clone()
     y[..., 0:2 * n:2] = u * c - v * s
@@ -368,30 +428,53 @@ def rope_qkv_cache(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch
                    slot_mapping: torch.Tensor, cache: torch.Tensor, koff: int, voff: int, num_heads: int,
                    num_kv_heads: int, dk: int, dv: int, block_size: int, freqs: torch.Tensor,
                    q_norm: Optional[torch.Tensor] = None, k_norm: Optional[torch.Tensor] = None, eps: float = 1e-5,
-                   v_freqs: Optional[torch.Tensor] = None) -> None:
+                   v_freqs: Optional[torch.Tensor] = None, *, bias_q: Optional[torch.Tensor] = None,
+                   bias_k: Optional[torch.Tensor] = None, bias_v: Optional[torch.Tensor] = None,
+                   norm_whole: bool = False, split_pairs: bool = False, mag: float = 1.0) -> None:
     """Queries, keys and values of a step from the fused projection to what attention reads, in one
     launch.  Per head: optional RMS norm over the head (weight [dk], plain), then interleaved rotary
     pairs (2i, 2i+1) on the first 2 * len(freqs) dimensions by position * freqs[i]; values are
     turned over 2 * len(v_freqs) dimensions when v_freqs is given.  q [T, H*dk] is rewritten in place;
     k [T, G*dk] and v [T, G*dv] go into the paged cache (slot -1: not written).  k = v = None: a layer
-    that reads another layer's pages.  Angles, norms and rotations in fp32, one rounding at the end."""
+    that reads another layer's pages.  Angles, norms and rotations in fp32, one rounding at the end.
+    The keyword forms (one launch of a workgroup per token): bias_q / bias_k / bias_v are added first;
+    norm_whole: ONE RMS norm over all of q's columns and one over all of k's (weights [H*dk], [G*dk]);
+    split_pairs: coordinate i pairs with i + len(freqs) instead of its neighbour; mag multiplies cos and sin."""
+    general = bias_q is not None or bias_k is not None or bias_v is not None or norm_whole or split_pairs or mag != 1.0
+    if _gpu(q) and general:
+        if v_freqs is not None:
+            raise ValueError("turned values come with the per-head form only")
+        ext().qkv_prep_cache(q, k, v, positions, slot_mapping, cache, int(koff), int(voff), num_heads, num_kv_heads, dk, dv,
+                             block_size, freqs, float(mag), bool(split_pairs), bias_q, bias_k, bias_v, q_norm, k_norm,
+                             float(eps), bool(norm_whole))
+        return
     if _gpu(q):
         ext().rope_qkv_cache(q, k, v, positions, slot_mapping, cache, int(koff), int(voff), num_heads, num_kv_heads,
                              dk, dv, block_size, freqs, q_norm, k_norm, float(eps), v_freqs)
         return
     T = q.shape[0]
 
-    def prep(x, heads, dim, norm_w, fr):
-        y = x.float().reshape(T, heads, dim)
-        if norm_w is not None:
+    def prep(x, heads, dim, norm_w, fr, bias):
+        y = x.float()
+        if bias is not None:
+            y = y + bias.float()
+        if norm_w is not None and norm_whole:
             y = _rms(y, eps) * norm_w.float()
-        return _rotate(y, positions, fr, 1.0) if fr is not None else y
+        y = y.reshape(T, heads, dim)
+        if norm_w is not None and not norm_whole:
+            y = _rms(y, eps) * norm_w.float()
+        if fr is None:
+            return y
+        if split_pairs:
+            n = fr.numel()
+            return torch.cat([_rotate_half(y[..., :2 * n], positions, fr, mag), y[..., 2 * n:]], dim=-1)
+        return _rotate(y, positions, fr, 1.0, mag)
 
-    q.copy_(prep(q, num_heads, dk, q_norm, freqs).reshape(T, -1).to(q.dtype))
+    q.copy_(prep(q, num_heads, dk, q_norm, freqs, bias_q).reshape(T, -1).to(q.dtype))
     if k is None:
         return
-    kk = prep(k, num_kv_heads, dk, k_norm, freqs).reshape(T, -1).to(k.dtype)
-    vv = prep(v, num_kv_heads, dv, None, v_freqs).reshape(T, -1).to(v.dtype)
+    kk = prep(k, num_kv_heads, dk, k_norm, freqs, bias_k).reshape(T, -1).to(k.dtype)
+    vv = prep(v, num_kv_heads, dv, None, v_freqs, bias_v).reshape(T, -1).to(v.dtype)
     kv_write(cache, kk, vv, slot_mapping, koff, voff, num_kv_heads, dk, dv, block_size)
 
 
@@ -580,23 +663,23 @@ def gated_norm(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, eps: float,
 
 
 # ----------------------------------------------------------------------------- latent attention
-def _rotate_half(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
+def _rotate_half(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor, mag: float = 1.0) -> torch.Tensor:
     """x fp32 [T, heads, 2n]: coordinate i pairs with i + n and the pair turns by pos * freqs[i]."""
     n = freqs.numel()
     ang = pos.to(torch.float32).view(-1, 1, 1) * freqs.float().view(1, 1, n)
-    c, s = torch.cos(ang), torch.sin(ang)
+    c, s = torch.cos(ang) * mag, torch.sin(ang) * mag
     u, v = x[..., :n], x[..., n:]
     return torch.cat([u * c - v * s, v * c + u * s], dim=-1)
 
 
 def latent_prep(dq: torch.Tensor, dkv: torch.Tensor, positions: torch.Tensor, slot_mapping: torch.Tensor,
                 cache: torch.Tensor, koff: int, rank: int, block_size: int, freqs: torch.Tensor,
-                q_norm: torch.Tensor, kv_norm: torch.Tensor, eps: float) -> torch.Tensor:
+                q_norm: torch.Tensor, kv_norm: torch.Tensor, eps: float, split_pairs: bool = True) -> torch.Tensor:
     """The two down-projections of a latent attention, from the fused projection to what the next
     steps read, in one launch.  dq [T, q_rank] (row-strided view): returns RMSNorm(dq) * q_norm as a
     new [T, q_rank].  dkv [T, rank + 2n]: the first `rank` columns RMS-normed times kv_norm, the last
-    2n (n = len(freqs)) turned in the half-split layout (i pairs with i + n) by position * freqs[i];
-    the row [latent | turned part] goes into the paged cache at `koff` as [BS, rank + 2n] (one shared
+    2n (n = len(freqs)) turned in the half-split layout (i pairs with i + n; split_pairs False: 2i with
+    2i + 1) by position * freqs[i]; the row [latent | turned part] goes into the paged cache at `koff` as [BS, rank + 2n] (one shared
     kv head; slot -1: not written).  Norms, angles and turns in fp32, one rounding at the end."""
     T, qr = dq.shape
     n = freqs.numel()
@@ -604,12 +687,13 @@ def latent_prep(dq: torch.Tensor, dkv: torch.Tensor, positions: torch.Tensor, sl
     if _gpu(dq):
         cq = torch.empty(T, qr, dtype=dq.dtype, device=dq.device)
         ext().latent_prep(cq, dq, dkv, positions, slot_mapping, cache, int(koff), int(rank), int(block_size), freqs,
-                          q_norm, kv_norm, float(eps))
+                          q_norm, kv_norm, float(eps), bool(split_pairs))
         return cq
     cq = (_rms(dq.float(), eps) * q_norm.float()).to(dq.dtype)
     d = dkv.float()
     c = _rms(d[:, :rank], eps) * kv_norm.float()
-    kr = _rotate_half(d[:, rank:].unsqueeze(1), positions, freqs).squeeze(1)
+    turn = _rotate_half if split_pairs else (lambda x, p, f: _rotate(x, p, f, 1.0))
+    kr = turn(d[:, rank:].unsqueeze(1), positions, freqs).squeeze(1)
     row = torch.cat([c, kr], dim=-1).to(cache.dtype)
     ok = slot_mapping >= 0
     slots = slot_mapping[ok]
@@ -619,17 +703,19 @@ def latent_prep(dq: torch.Tensor, dkv: torch.Tensor, positions: torch.Tensor, sl
 
 
 def rope_half_into(out: torch.Tensor, x: torch.Tensor, positions: torch.Tensor, heads: int, x_dim: int, x_col: int,
-                   out_dim: int, out_col: int, freqs: torch.Tensor) -> None:
+                   out_dim: int, out_col: int, freqs: torch.Tensor, split_pairs: bool = True) -> None:
     """Per token and head: the 2n columns of x's head (x [T, heads*x_dim], from column x_col of the head)
-    turned in the half-split layout by position * freqs[i], written to columns out_col.. of the same
-    head in out [T, heads*out_dim].  fp32 inside."""
+    turned in the half-split layout (split_pairs False: as neighbouring pairs) by position * freqs[i],
+    written to columns out_col.. of the same head in out [T, heads*out_dim].  fp32 inside."""
     n = freqs.numel()
     if _gpu(x):
-        ext().rope_half_into(out, x, positions, int(heads), int(x_dim), int(x_col), int(out_dim), int(out_col), freqs)
+        ext().rope_half_into(out, x, positions, int(heads), int(x_dim), int(x_col), int(out_dim), int(out_col), freqs,
+                             bool(split_pairs))
         return
     T = x.shape[0]
     part = x.reshape(T, heads, x_dim)[:, :, x_col:x_col + 2 * n].float()
-    out.view(T, heads, out_dim)[:, :, out_col:out_col + 2 * n] = _rotate_half(part, positions, freqs).to(out.dtype)
+    turned = _rotate_half(part, positions, freqs) if split_pairs else _rotate(part, positions, freqs, 1.0)
+    out.view(T, heads, out_dim)[:, :, out_col:out_col + 2 * n] = turned.to(out.dtype)
 
 
 LATENT_TARGET_WAVES = 1024  # waves that fill the 256 CUs one deep: single-token steps split their keys up to this
@@ -640,9 +726,11 @@ LATENT_WIDE_FORM = os.environ.get("MXS_LATENT_WIDE_FORM", "auto")
 
 def latent_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.Tensor, qsl: torch.Tensor,
                      seq_lens: torch.Tensor, koff: int, num_heads: int, dk: int, rank: int, block_size: int, scale: float,
-                     max_query_len: int = 0, max_seq_len: int = 0, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     max_query_len: int = 0, max_seq_len: int = 0, sink: Optional[torch.Tensor] = None,
+                     window: int = 0) -> torch.Tensor:
     """Softmax attention of every head over the same cached rows [latent | rotated part] (dk entries a
-    row at `koff`, written by latent_prep), causal; the values are the rows' first `rank` entries.
+    row at `koff`, written by latent_prep), causal, within the last `window` positions when window > 0;
+    the values are the rows' first `rank` entries.
     q [T, H*dk] (the folded queries) -> the weighted latents [T, H*rank]; scores and weights fp32; sink as
     in window_attention.  bf16 on the GPU with dk a multiple of 8 up to 576 and rank a multiple of 16 up
     to 512 runs the matrix-core kernel; a step of few rows splits each row's keys over several waves
@@ -653,31 +741,32 @@ def latent_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
         S = seq_lens.numel()
         mq = max(1, min(int(max_query_len) or T, T))
         tiles = S * (-(-mq * num_heads // 16))
-        blocks = max(1, -(-(int(max_seq_len) or 16) // 16))
+        span = min(int(max_seq_len) or 16, int(window) + 15) if window > 0 else (int(max_seq_len) or 16)
+        blocks = max(1, -(-span // 16))
         nsplit = max(1, min(16, LATENT_TARGET_WAVES // max(tiles, 1), blocks // 2))
         out = torch.empty(T, num_heads * rank, dtype=q.dtype, device=q.device)
         part = (torch.empty(T * num_heads * nsplit * (rank + 4), dtype=torch.float32, device=q.device)
                 if nsplit > 1 else None)
         if ext().latent_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), num_heads, dk, rank, block_size,
                                   float(scale), mq, sink, nsplit, part,
-                                  LATENT_WIDE_FORM != "single"):
+                                  LATENT_WIDE_FORM != "single", int(window)):
             return out
     return window_attention(q, cache, block_tables, qsl, seq_lens, koff, koff, num_heads, 1, dk, rank, block_size, scale,
-                            0, 0, max_query_len, sink=sink, v_stride=dk)
+                            int(window), 0, max_query_len, sink=sink, v_stride=dk)
 
 
 # ----------------------------------------------------------------------------- routed experts
-def route_topk(logits: torch.Tensor, k: int, renorm: bool = False) -> tuple:
-    """Sigmoid router: scores = sigmoid(logits) (fp32 [T, E]); the k largest per token (ties: the
-    lower index first), their scores as weights (renorm: divided by their sum).
+def route_topk(logits: torch.Tensor, k: int, renorm: bool = False, softmax: bool = False) -> tuple:
+    """Router: scores = sigmoid(logits), or softmax over all experts (fp32 [T, E]); the k largest per
+    token (ties: the lower index first), their scores as weights (renorm: divided by their sum).
     -> (weights fp32 [T, k], ids int32 [T, k])."""
     T, E = logits.shape
     if _gpu(logits):
         w = torch.empty(T, k, dtype=torch.float32, device=logits.device)
         ids = torch.empty(T, k, dtype=torch.int32, device=logits.device)
-        ext().route_topk(w, ids, logits, bool(renorm))
+        ext().route_topk(w, ids, logits, bool(renorm), bool(softmax))
         return w, ids
-    s = torch.sigmoid(logits.float())
+    s = torch.softmax(logits.float(), dim=-1) if softmax else torch.sigmoid(logits.float())
     order = torch.argsort(s, dim=-1, descending=True, stable=True)[:, :k]
     w = torch.gather(s, 1, order)
     if renorm:
@@ -717,47 +806,57 @@ def expert_align(ids: torch.Tensor, num_experts: int) -> tuple:
     return offs.to(torch.int32), inv.to(torch.int32)
 
 
-def gather_scaled(h: torch.Tensor, weights: torch.Tensor, inv: torch.Tensor) -> torch.Tensor:
+def gather_scaled(h: torch.Tensor, weights: Optional[torch.Tensor], inv: torch.Tensor, k: int = 0) -> torch.Tensor:
     """xs[inv[p]] = weights[p] * h[p // k] for every pair p (weights fp32 [T, k]): the experts' inputs,
-    sorted by expert, each already times its routing weight (product in fp32, rounded once)."""
-    T, k = weights.shape
+    sorted by expert, each already times its routing weight (product in fp32, rounded once).
+    weights None (then k says how many pairs a token has): the rows themselves."""
+    T = h.shape[0]
+    k = int(k) if weights is None else weights.shape[1]
     xs = torch.empty(T * k, h.shape[1], dtype=h.dtype, device=h.device)
     if _gpu(h):
-        ext().gather_scaled(xs, h, weights, inv)
+        ext().gather_scaled(xs, h, weights, inv, k)
         return xs
-    rows = (h.float().unsqueeze(1) * weights.float().unsqueeze(2)).reshape(T * k, -1).to(h.dtype)
+    if weights is None:
+        rows = h.unsqueeze(1).expand(T, k, h.shape[1]).reshape(T * k, -1)
+    else:
+        rows = (h.float().unsqueeze(1) * weights.float().unsqueeze(2)).reshape(T * k, -1).to(h.dtype)
     xs[inv.long()] = rows
     return xs
 
 
-def spread_scaled(h: torch.Tensor, weights: torch.Tensor, ids: torch.Tensor, num_experts: int) -> torch.Tensor:
+def spread_scaled(h: torch.Tensor, weights: Optional[torch.Tensor], ids: torch.Tensor, num_experts: int) -> torch.Tensor:
     """[E, T, W]: row (e, t) = weights[t, j] * h[t] where ids[t, j] = e, zeros for the experts a token
-    did not choose (the experts' inputs for a batched product over all experts, no sorting)."""
-    T, k = weights.shape
+    did not choose (the experts' inputs for a batched product over all experts, no sorting).
+    weights None: the chosen rows are h[t] itself."""
+    T, k = ids.shape
     if _gpu(h):
         xs = torch.empty(num_experts, T, h.shape[1], dtype=h.dtype, device=h.device)
         ext().spread_scaled(xs, h, weights, ids)
         return xs
     cw = torch.zeros(T, num_experts, dtype=torch.float32)
-    cw.scatter_(1, ids.long(), weights.float())
+    cw.scatter_(1, ids.long(), torch.ones(T, k) if weights is None else weights.float())
     return (cw.t().unsqueeze(2) * h.float().unsqueeze(0)).to(h.dtype)
 
 
 def expert_combine(ys: torch.Tensor, index: Optional[torch.Tensor], k: int, T: int, extra: Optional[torch.Tensor] = None,
-                   row_stride: int = 0) -> torch.Tensor:
+                   row_stride: int = 0, weights: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out[t] = sum_j ys[index[t*k + j]] (+ extra[t]); index None: row j*row_stride + t (the k slabs
-    of a [k, T, W] stack).  Summed in fp32, rounded once."""
+    of a [k, T, W] stack).  weights (fp32 [T, k]): row j of token t enters times weights[t, j] (routing
+    weights on the experts' outputs).  Summed in fp32, rounded once."""
     W = ys.shape[-1]
     y2 = ys.reshape(-1, W)
     if _gpu(ys):
         out = torch.empty(T, W, dtype=ys.dtype, device=ys.device)
-        ext().expert_combine(out, y2, index, int(k), extra, int(row_stride))
+        ext().expert_combine(out, y2, index, int(k), extra, int(row_stride), weights)
         return out
     if index is None:
         idx = (torch.arange(k).view(1, k) * row_stride + torch.arange(T).view(T, 1)).reshape(-1)
     else:
         idx = index.long()
-    acc = y2[idx].float().view(T, k, W).sum(1)
+    rows = y2[idx].float().view(T, k, W)
+    if weights is not None:
+        rows = rows * weights.float().view(T, k, 1)
+    acc = rows.sum(1)
     if extra is not None:
         acc = acc + extra.float()
     return acc.to(ys.dtype)
