@@ -9,7 +9,17 @@
 
 namespace mxs {
 void launch_resid_update(float*, const void*, long, const void*, const void*, long, const void*, const void*, int,
-                         const void*, void*, int, int, float, float, float, bool, hipStream_t);
+                         const void*, void*, int, int, float, float, float, float, bool, hipStream_t);
+void launch_embed_normed(float*, void*, const int64_t*, const void*, const void*, int, int, long, float, float, bool,
+                         hipStream_t);
+bool launch_depth_mix(float*, long, int, const float*, void*, int, int, bool, hipStream_t);
+void launch_xielu(void*, const void*, long, const float*, bool, hipStream_t);
+void launch_qkv_prep_cache(void*, long, const void*, long, const void*, long, const int64_t*, const int64_t*, void*, long,
+                           int, int, int, int, int, int, int, int, const float*, int, float, bool, const void*, const void*,
+                           const void*, const void*, const void*, float, int, bool, hipStream_t);
+bool launch_talking_attention(void*, const void*, long, const void*, long, const int*, int, const int*, const int*, int,
+                              int, int, int, int, int, int, int, int, float, int, int, int, const float*, const float*, bool,
+                              hipStream_t);
 void launch_cast_into(void*, long, const float*, int, int, bool, hipStream_t);
 void launch_relu_sq(void*, const void*, long, bool, hipStream_t);
 void launch_softcap(float*, const void*, long, int, int, float, bool, hipStream_t);
@@ -36,17 +46,18 @@ void launch_gated_norm(void*, long, const float*, const void*, long, const void*
                        float, bool, hipStream_t);
 bool launch_column_scan(const ScanArgs&, int, bool, bool, hipStream_t);
 bool launch_latent_attention(void*, float*, const void*, long, const void*, long, const int*, int, const int*, const int*,
-                             int, int, int, int, int, int, int, float, int, const float*, int, bool, hipStream_t);
+                             int, int, int, int, int, int, int, float, int, const float*, int, bool, int, hipStream_t);
 void launch_latent_prep(void*, const void*, long, const void*, long, const int64_t*, const int64_t*, void*, long, int, int,
-                        int, int, int, int, const float*, const void*, const void*, float, bool, hipStream_t);
+                        int, int, int, int, const float*, const void*, const void*, float, bool, bool, hipStream_t);
 void launch_rope_half_into(void*, long, const void*, long, const int64_t*, int, int, int, int, int, int, const float*, int,
-                           bool, hipStream_t);
-void launch_route_topk(float*, int*, const float*, int, int, int, bool, hipStream_t);
+                           bool, bool, hipStream_t);
+void launch_route_topk(float*, int*, const float*, int, int, int, bool, bool, hipStream_t);
 void launch_capped_glu(void*, const void*, long, int, int, float, float, bool, hipStream_t);
 bool launch_expert_align(int*, int*, const int*, int, int, hipStream_t);
 void launch_gather_scaled(void*, const void*, long, const float*, const int*, int, int, int, bool, hipStream_t);
 void launch_spread_scaled(void*, const void*, long, const float*, const int*, int, int, int, int, bool, hipStream_t);
-void launch_expert_combine(void*, const void*, const int*, int, int, long, const void*, long, int, bool, hipStream_t);
+void launch_expert_combine(void*, const void*, const int*, int, int, long, const void*, long, int, const float*, bool,
+                           hipStream_t);
 }  // namespace mxs
 
 namespace {
@@ -87,18 +98,18 @@ float* f32(const at::Tensor& t, const char* name) {
 }
 
 void resid_update(at::Tensor x, OptT a, OptT wa, OptT b, OptT wb, OptT bias, bool assign, OptT norm_w, OptT h,
-                  double eps, double a_scale, double w_offset) {
+                  double eps, double a_scale, double w_offset, double wa_offset) {
   float* xp = f32(x, "x");
   TORCH_CHECK(x.dim() == 2, "x: [T, W]");
   const int64_t T = x.size(0), W = x.size(1);
-  const at::Tensor* any = a.has_value() ? &*a : (norm_w.has_value() ? &*norm_w : nullptr);
+  const at::Tensor* any = a.has_value() ? &*a : (norm_w.has_value() ? &*norm_w : (h.has_value() ? &*h : nullptr));
   if (any == nullptr || T == 0) return;
   const bool bf = is_bf(*any);
   const void* ap = a.has_value() ? mat(*a, bf, T, W, "a") : nullptr;
   const void* bp = b.has_value() ? mat(*b, bf, T, W, "b") : nullptr;
   TORCH_CHECK(!b.has_value() || (a.has_value() && wa.has_value() && wb.has_value()), "two branches need both weights");
   TORCH_CHECK(!assign || a.has_value(), "assign needs a");
-  TORCH_CHECK(norm_w.has_value() == h.has_value(), "norm_w and h go together");
+  TORCH_CHECK(!norm_w.has_value() || h.has_value(), "norm_w needs h (h alone: the updated x, cast)");
   void* hp = nullptr;
   if (h.has_value()) {
     TORCH_CHECK(h->is_cuda() && h->is_contiguous() && h->dim() == 2 && h->size(0) == T && h->size(1) == W &&
@@ -108,8 +119,8 @@ void resid_update(at::Tensor x, OptT a, OptT wa, OptT b, OptT wb, OptT bias, boo
   mxs::launch_resid_update(xp, ap, a.has_value() ? a->stride(0) : 0, vec(wa, bf, W, "wa"), bp,
                            b.has_value() ? b->stride(0) : 0, vec(wb, bf, W, "wb"), vec(bias, bf, W, "bias"), assign,
                            vec(norm_w, bf, W, "norm_w"), hp, static_cast<int>(T), static_cast<int>(W),
-                           static_cast<float>(eps), static_cast<float>(a_scale), static_cast<float>(w_offset), bf,
-                           stream());
+                           static_cast<float>(eps), static_cast<float>(a_scale), static_cast<float>(w_offset),
+                           static_cast<float>(wa_offset), bf, stream());
 }
 
 void cast_into(at::Tensor dst, at::Tensor x) {
@@ -443,7 +454,7 @@ const int64_t* i64c(const at::Tensor& t, int64_t n, const char* name) {
 
 void latent_prep(at::Tensor cq, at::Tensor dq, at::Tensor dkv, at::Tensor positions, at::Tensor slots, at::Tensor cache,
                  int64_t koff, int64_t rank, int64_t bs, at::Tensor freqs, at::Tensor q_norm, at::Tensor kv_norm,
-                 double eps) {
+                 double eps, bool split_pairs) {
   const bool bf = is_bf(dq);
   const int64_t T = dq.size(0), qr = dq.size(1), nf = freqs.numel(), dk = rank + 2 * nf;
   TORCH_CHECK(rank >= 1 && bs >= 1, "rank and block size must be positive");
@@ -455,15 +466,16 @@ void latent_prep(at::Tensor cq, at::Tensor dq, at::Tensor dkv, at::Tensor positi
                           static_cast<int>(T), static_cast<int>(koff), static_cast<int>(qr), static_cast<int>(rank),
                           static_cast<int>(nf), static_cast<int>(bs), f32(freqs, "freqs"),
                           vec(OptT(q_norm), bf, qr, "q_norm"), vec(OptT(kv_norm), bf, rank, "kv_norm"),
-                          static_cast<float>(eps), bf, stream());
+                          static_cast<float>(eps), split_pairs, bf, stream());
 }
 
 // The matrix-core latent attention (bf16).  Returns false when the sizes are not the kernel's: nothing
 // was launched and the caller runs window_attention with strided value rows instead.
 bool latent_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor block_tables, at::Tensor qsl,
                       at::Tensor seq_lens, int64_t koff, int64_t H, int64_t dk, int64_t rank, int64_t bs, double scale,
-                      int64_t max_query_len, OptT sink, int64_t nsplit, OptT part, bool pair) {
+                      int64_t max_query_len, OptT sink, int64_t nsplit, OptT part, bool pair, int64_t window) {
   if (!is_bf(q)) return false;
+  TORCH_CHECK(window >= 0 && window < (1LL << 30), "window out of range");
   const float* sinkp = nullptr;
   if (sink.has_value()) {
     sinkp = f32(*sink, "sink");
@@ -486,11 +498,12 @@ bool latent_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor
       block_tables.data_ptr<int>(), static_cast<int>(block_tables.stride(0)), i32(qsl, S + 1, "qsl"),
       i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(koff), static_cast<int>(H),
       static_cast<int>(dk), static_cast<int>(rank), static_cast<int>(bs), static_cast<float>(scale),
-      static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(max_query_len, T))), sinkp, static_cast<int>(nsplit), pair, stream());
+      static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(max_query_len, T))), sinkp, static_cast<int>(nsplit), pair,
+      static_cast<int>(window), stream());
 }
 
 void rope_half_into(at::Tensor out, at::Tensor x, at::Tensor positions, int64_t heads, int64_t x_dim, int64_t x_col,
-                    int64_t out_dim, int64_t out_col, at::Tensor freqs) {
+                    int64_t out_dim, int64_t out_col, at::Tensor freqs, bool split_pairs) {
   const bool bf = is_bf(x);
   const int64_t T = x.size(0), nf = freqs.numel();
   TORCH_CHECK(x_col >= 0 && out_col >= 0 && x_col + 2 * nf <= x_dim && out_col + 2 * nf <= out_dim,
@@ -499,17 +512,17 @@ void rope_half_into(at::Tensor out, at::Tensor x, at::Tensor positions, int64_t 
                              mat(x, bf, T, heads * x_dim, "x"), x.stride(0), i64c(positions, T, "positions"),
                              static_cast<int>(T), static_cast<int>(heads), static_cast<int>(x_dim), static_cast<int>(x_col),
                              static_cast<int>(out_dim), static_cast<int>(out_col), f32(freqs, "freqs"), static_cast<int>(nf),
-                             bf, stream());
+                             split_pairs, bf, stream());
 }
 
-void route_topk(at::Tensor w, at::Tensor ids, at::Tensor logits, bool renorm) {
+void route_topk(at::Tensor w, at::Tensor ids, at::Tensor logits, bool renorm, bool softmax) {
   const float* lp = f32(logits, "logits");
   TORCH_CHECK(logits.dim() == 2 && w.dim() == 2 && ids.dim() == 2, "logits [T, E], w / ids [T, k]");
   const int64_t T = logits.size(0), E = logits.size(1), k = w.size(1);
   TORCH_CHECK(k >= 1 && k <= E && w.size(0) == T && ids.size(0) == T && ids.size(1) == k, "1 <= k <= E; w, ids [T, k]");
   TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kInt && ids.is_contiguous(), "ids: contiguous int32");
   mxs::launch_route_topk(f32(w, "w"), ids.data_ptr<int>(), lp, static_cast<int>(T), static_cast<int>(E),
-                         static_cast<int>(k), renorm, stream());
+                         static_cast<int>(k), renorm, softmax, stream());
 }
 
 void capped_glu(at::Tensor out, at::Tensor gu, double limit, double alpha) {
@@ -532,44 +545,157 @@ void expert_align(at::Tensor offs, at::Tensor inv, at::Tensor ids, int64_t E) {
               "expert_align: more experts than the kernel's counters hold");
 }
 
-void gather_scaled(at::Tensor xs, at::Tensor h, at::Tensor w, at::Tensor inv) {
+void gather_scaled(at::Tensor xs, at::Tensor h, OptT w, at::Tensor inv, int64_t k) {
   const bool bf = is_bf(h);
-  TORCH_CHECK(w.dim() == 2 && h.dim() == 2 && w.size(0) == h.size(0), "h [T, W], w [T, k]");
-  const int64_t T = h.size(0), W = h.size(1), k = w.size(1);
+  TORCH_CHECK(h.dim() == 2 && k >= 1, "h [T, W], k >= 1");
+  const int64_t T = h.size(0), W = h.size(1);
+  const float* wp = nullptr;
+  if (w.has_value()) {
+    TORCH_CHECK(w->dim() == 2 && w->size(0) == T && w->size(1) == k, "w [T, k]");
+    wp = f32(*w, "w");
+  }
   TORCH_CHECK(xs.is_cuda() && xs.is_contiguous() && xs.dim() == 2 && xs.size(0) == T * k && xs.size(1) == W &&
               is_bf(xs) == bf, "xs: contiguous [T*k, W]");
   // inv comes from expert_align over the same pairs: a permutation of 0 .. T*k-1
-  mxs::launch_gather_scaled(xs.data_ptr(), mat(h, bf, T, W, "h"), h.stride(0), f32(w, "w"), i32(inv, T * k, "inv"),
+  mxs::launch_gather_scaled(xs.data_ptr(), mat(h, bf, T, W, "h"), h.stride(0), wp, i32(inv, T * k, "inv"),
                             static_cast<int>(T * k), static_cast<int>(k), static_cast<int>(W), bf, stream());
 }
 
-void spread_scaled(at::Tensor xs, at::Tensor h, at::Tensor w, at::Tensor ids) {
+void spread_scaled(at::Tensor xs, at::Tensor h, OptT w, at::Tensor ids) {
   const bool bf = is_bf(h);
-  TORCH_CHECK(w.dim() == 2 && h.dim() == 2 && w.size(0) == h.size(0) && xs.dim() == 3, "h [T, W], w [T, k], xs [E, T, W]");
-  const int64_t T = h.size(0), W = h.size(1), k = w.size(1), E = xs.size(0);
+  TORCH_CHECK(ids.dim() == 2 && h.dim() == 2 && ids.size(0) == h.size(0) && xs.dim() == 3, "h [T, W], ids [T, k], xs [E, T, W]");
+  const int64_t T = h.size(0), W = h.size(1), k = ids.size(1), E = xs.size(0);
+  const float* wp = nullptr;
+  if (w.has_value()) {
+    TORCH_CHECK(w->dim() == 2 && w->size(0) == T && w->size(1) == k, "w [T, k]");
+    wp = f32(*w, "w");
+  }
   TORCH_CHECK(xs.is_cuda() && xs.is_contiguous() && xs.size(1) == T && xs.size(2) == W && is_bf(xs) == bf,
               "xs: contiguous [E, T, W]");
   TORCH_CHECK(E <= 65535, "more experts than a grid dimension holds");
-  mxs::launch_spread_scaled(xs.data_ptr(), mat(h, bf, T, W, "h"), h.stride(0), f32(w, "w"), i32(ids, T * k, "ids"),
+  mxs::launch_spread_scaled(xs.data_ptr(), mat(h, bf, T, W, "h"), h.stride(0), wp, i32(ids, T * k, "ids"),
                             static_cast<int>(T), static_cast<int>(E), static_cast<int>(k), static_cast<int>(W), bf,
                             stream());
 }
 
-void expert_combine(at::Tensor out, at::Tensor ys, OptT index, int64_t k, OptT extra, int64_t row_stride) {
+void expert_combine(at::Tensor out, at::Tensor ys, OptT index, int64_t k, OptT extra, int64_t row_stride, OptT weights) {
   const bool bf = is_bf(ys);
   TORCH_CHECK(ys.is_cuda() && ys.is_contiguous() && ys.dim() == 2 && out.is_cuda() && out.is_contiguous() &&
               out.dim() == 2 && out.size(1) == ys.size(1) && is_bf(out) == bf, "ys [R, W], out [T, W]");
   const int64_t T = out.size(0), W = out.size(1), R = ys.size(0);
   const int* ip = nullptr;
   if (index.has_value()) {
-    ip = i32(*index, T * k, "index");  // entries are rows of ys: expert_align's places, < T*k <= R
+    ip = i32(*index, T * k, "index");  // entries are rows of ys: expert_align's places (< T*k), or expert * T + t (< R)
     TORCH_CHECK(T * k <= R, "index reaches past ys");
   } else {
     TORCH_CHECK(k >= 1 && row_stride >= T && (k - 1) * row_stride + T <= R, "the k slabs reach past ys");
   }
   const void* ep = extra.has_value() ? mat(*extra, bf, T, W, "extra") : nullptr;
+  const float* wp = nullptr;
+  if (weights.has_value()) {
+    TORCH_CHECK(weights->numel() == T * k, "weights: fp32 [T, k]");
+    wp = f32(*weights, "weights");
+  }
   mxs::launch_expert_combine(out.data_ptr(), ys.data_ptr(), ip, static_cast<int>(T), static_cast<int>(k), row_stride, ep,
-                             extra.has_value() ? extra->stride(0) : 0, static_cast<int>(W), bf, stream());
+                             extra.has_value() ? extra->stride(0) : 0, static_cast<int>(W), wp, bf, stream());
+}
+
+void embed_normed(at::Tensor out, OptT h, at::Tensor ids, at::Tensor table, at::Tensor w, double eps, double w_offset) {
+  float* op = f32(out, "out");
+  TORCH_CHECK(table.is_cuda() && table.dim() == 2 && table.is_contiguous(), "table: contiguous [vocab, W]");
+  const bool bf = is_bf(table);
+  const int64_t T = ids.numel(), W = table.size(1);
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == T && out.size(1) == W, "out: fp32 [T, W]");
+  void* hp = nullptr;
+  if (h.has_value()) {
+    TORCH_CHECK(h->is_cuda() && h->is_contiguous() && h->dim() == 2 && h->size(0) == T && h->size(1) == W && is_bf(*h) == bf,
+                "h: contiguous [T, W] of the table's dtype");
+    hp = h->data_ptr();
+  }
+  mxs::launch_embed_normed(op, hp, i64c(ids, T, "ids"), table.data_ptr(), vec(OptT(w), bf, W, "w"), static_cast<int>(T),
+                           static_cast<int>(W), table.size(0), static_cast<float>(eps), static_cast<float>(w_offset), bf,
+                           stream());
+}
+
+void depth_mix(at::Tensor hist, int64_t n, at::Tensor coeffs, OptT h) {
+  float* hp = f32(hist, "hist");
+  TORCH_CHECK(hist.dim() == 3 && n >= 1 && n < hist.size(0), "hist: fp32 [L, T, W], 1 <= n < L");
+  const int64_t T = hist.size(1), W = hist.size(2);
+  const float* cp = f32(coeffs, "coeffs");
+  TORCH_CHECK(coeffs.numel() == n, "coeffs: fp32 [n]");
+  void* op = nullptr;
+  bool bf = false;
+  if (h.has_value()) {
+    TORCH_CHECK(h->is_cuda() && h->is_contiguous() && h->dim() == 2 && h->size(0) == T && h->size(1) == W, "h: contiguous [T, W]");
+    bf = is_bf(*h);
+    op = h->data_ptr();
+  }
+  TORCH_CHECK(mxs::launch_depth_mix(hp, T * W, static_cast<int>(n), cp, op, static_cast<int>(T), static_cast<int>(W), bf,
+                                    stream()), "depth_mix: more slabs than the kernel's coefficient table holds");
+}
+
+void xielu(at::Tensor out, at::Tensor x, at::Tensor ab) {
+  TORCH_CHECK(x.is_cuda() && x.is_contiguous() && out.is_cuda() && out.is_contiguous() && out.numel() == x.numel() &&
+              out.scalar_type() == x.scalar_type(), "xielu: contiguous tensors of one dtype");
+  const float* ap = f32(ab, "ab");
+  TORCH_CHECK(ab.numel() == 2, "ab: fp32 [2]");
+  mxs::launch_xielu(out.data_ptr(), x.data_ptr(), x.numel(), ap, is_bf(x), stream());
+}
+
+// Biases, q / k norms (norm_whole: one over all of a row's heads), rotary turn, q in place, k and v into the pages.
+void qkv_prep_cache(at::Tensor q, OptT k, OptT v, at::Tensor positions, at::Tensor slots, at::Tensor cache, int64_t koff,
+                    int64_t voff, int64_t H, int64_t G, int64_t dk, int64_t dv, int64_t bs, at::Tensor freqs, double mag,
+                    bool split_pairs, OptT bq, OptT bk, OptT bv, OptT q_norm, OptT k_norm, double eps, bool norm_whole) {
+  const bool bf = is_bf(q);
+  const int64_t T = q.size(0);
+  TORCH_CHECK(k.has_value() == v.has_value(), "k and v go together");
+  TORCH_CHECK(H >= 1 && G >= 1 && H <= 4096 && G <= 4096 && dk >= 1 && bs >= 1, "head counts / sizes out of range");
+  const void *kp = nullptr, *vp = nullptr;
+  if (k.has_value()) {
+    check_cache(cache, bf, koff, voff, G, dk, dv, bs);
+    kp = mat(*k, bf, T, G * dk, "k");
+    vp = mat(*v, bf, T, G * dv, "v");
+  }
+  const int64_t nf = freqs.numel();
+  TORCH_CHECK(2 * nf <= dk, "more rotary pairs than the head has dimensions");
+  const int64_t nq = norm_whole ? H * dk : dk, nk = norm_whole ? G * dk : dk;
+  mxs::launch_qkv_prep_cache(const_cast<void*>(mat(q, bf, T, H * dk, "q")), q.stride(0), kp, k.has_value() ? k->stride(0) : 0,
+                             vp, v.has_value() ? v->stride(0) : 0, i64c(positions, T, "positions"),
+                             i64c(slots, T, "slot_mapping"), cache.data_ptr(), cache.stride(0), static_cast<int>(T),
+                             static_cast<int>(koff), static_cast<int>(voff), static_cast<int>(H), static_cast<int>(G),
+                             static_cast<int>(dk), static_cast<int>(dv), static_cast<int>(bs), f32(freqs, "freqs"),
+                             static_cast<int>(nf), static_cast<float>(mag), split_pairs, vec(bq, bf, H * dk, "bias_q"),
+                             vec(bk, bf, G * dk, "bias_k"), vec(bv, bf, G * dv, "bias_v"), vec(q_norm, bf, nq, "q_norm"),
+                             vec(k_norm, bf, nk, "k_norm"), static_cast<float>(eps), norm_whole ? 2 : 1, bf, stream());
+}
+
+void talking_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor block_tables, at::Tensor qsl,
+                       at::Tensor seq_lens, int64_t koff, int64_t voff, int64_t H, int64_t G, int64_t dk, int64_t dv,
+                       int64_t bs, double scale, int64_t window, int64_t keep, int64_t max_query_len, OptT sink,
+                       at::Tensor talk) {
+  const bool bf = is_bf(q);
+  const float* sinkp = nullptr;
+  if (sink.has_value()) {
+    sinkp = f32(*sink, "sink");
+    TORCH_CHECK(sink->numel() == H, "sink: fp32 [H]");
+  }
+  const float* tp = f32(talk, "talk");
+  TORCH_CHECK(talk.numel() == H * H, "talk: fp32 [H, H]");
+  const int64_t T = q.size(0), S = seq_lens.numel();
+  check_cache(cache, bf, koff, voff, G, dk, dv, bs);
+  TORCH_CHECK(G >= 1 && H % G == 0, "query heads must divide over kv heads");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == T && out.size(1) == H * dv &&
+              is_bf(out) == bf, "out: [T, H*dv]");
+  TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == at::kInt && block_tables.dim() == 2 &&
+              block_tables.size(0) >= S && block_tables.stride(1) == 1, "block_tables: int32 [S, max_blocks]");
+  const bool ok = mxs::launch_talking_attention(
+      out.data_ptr(), mat(q, bf, T, H * dk, "q"), q.stride(0), cache.data_ptr(), cache.stride(0),
+      block_tables.data_ptr<int>(), static_cast<int>(block_tables.stride(0)), i32(qsl, S + 1, "qsl"),
+      i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(koff),
+      static_cast<int>(voff), static_cast<int>(H), static_cast<int>(G), static_cast<int>(dk), static_cast<int>(dv),
+      static_cast<int>(bs), static_cast<float>(scale), static_cast<int>(window), static_cast<int>(keep),
+      static_cast<int>(std::min<int64_t>(max_query_len, T)), sinkp, tp, bf, stream());
+  TORCH_CHECK(ok, "talking_attention: more heads or wider heads than the kernel's LDS tables hold");
 }
 
 }  // namespace
@@ -602,4 +728,9 @@ PYBIND11_MODULE(_M, m) {
   m.def("gather_scaled", &gather_scaled);
   m.def("spread_scaled", &spread_scaled);
   m.def("expert_combine", &expert_combine);
+  m.def("embed_normed", &embed_normed);
+  m.def("depth_mix", &depth_mix);
+  m.def("xielu", &xielu);
+  m.def("qkv_prep_cache", &qkv_prep_cache);
+  m.def("talking_attention", &talking_attention);
 }

@@ -6,14 +6,15 @@
 namespace mxs {
 
 // x (fp32, in place) <- x + d | d, d built from up to two branch outputs (each optionally RMS-normed
-// over the row with its weight, then averaged) and a bias row; h <- RMSNorm(x) * norm_w when asked.
+// over the row with its weight, then averaged) and a bias row; h <- RMSNorm(x) * norm_w when asked, or
+// h <- x itself (rounded to T) when h is given without norm_w.
 template <typename T>
 __global__ void __launch_bounds__(256) resid_update_kernel(float* __restrict__ x, const T* __restrict__ a, long a_stride,
                                                            const T* __restrict__ wa, const T* __restrict__ b,
                                                            long b_stride, const T* __restrict__ wb,
                                                            const T* __restrict__ bias, int assign,
                                                            const T* __restrict__ norm_w, T* __restrict__ h, int W,
-                                                           float eps, float a_scale, float w_offset) {
+                                                           float eps, float a_scale, float w_offset, float wa_offset) {
   __shared__ float scratch[16];
   const long row = blockIdx.x;
   float* xr = x + row * W;
@@ -35,12 +36,13 @@ __global__ void __launch_bounds__(256) resid_update_kernel(float* __restrict__ x
     float xv = xr[c];
     if (ar) {
       float d = ldf(ar + c) * a_scale;
-      if (wa) d = d * ra * ldf(wa + c);
+      if (wa) d = d * ra * (wa_offset + ldf(wa + c));
       if (br) d = 0.5f * (d + ldf(br + c) * rb * ldf(wb + c));
       if (bias) d += ldf(bias + c);
       xv = assign ? d : xv + d;
       xr[c] = xv;
     }
+    if (h && !norm_w) stf(h + row * W + c, xv);
     ss += xv * xv;
   }
   if (norm_w == nullptr) return;
@@ -163,11 +165,11 @@ __global__ void __launch_bounds__(256) kv_write_kernel(T* __restrict__ cache, lo
 
 void launch_resid_update(float* x, const void* a, long a_stride, const void* wa, const void* b, long b_stride,
                          const void* wb, const void* bias, int assign, const void* norm_w, void* h, int rows, int W,
-                         float eps, float a_scale, float w_offset, bool bf, hipStream_t st) {
+                         float eps, float a_scale, float w_offset, float wa_offset, bool bf, hipStream_t st) {
   if (rows == 0) return;
   MIX_DISPATCH(bf, hipLaunchKernelGGL(resid_update_kernel<T>, dim3(rows), dim3(256), 0, st, x, (const T*)a, a_stride,
                                       (const T*)wa, (const T*)b, b_stride, (const T*)wb, (const T*)bias, assign,
-                                      (const T*)norm_w, (T*)h, W, eps, a_scale, w_offset));
+                                      (const T*)norm_w, (T*)h, W, eps, a_scale, w_offset, wa_offset));
   MXS_CHECK_LAUNCH();
 }
 

@@ -3,8 +3,8 @@
 // first `rank` entries.  Prompt chunks and single decoded tokens run the same kernel.
 //
 // The rows of a sequence's step are its (token, head) pairs, flattened; a wave owns 16 consecutive
-// rows and walks the 16-key cache blocks that its rows see (causal), or one of `nsplit` stretches of
-// them.  No workgroup barriers: the four waves of a workgroup are independent.  Per block, with
+// rows and walks the 16-key cache blocks that its rows see (causal; with window > 0 only the last
+// `window` positions of each row), or one of `nsplit` stretches of them.  No workgroup barriers: the four waves of a workgroup are independent.  Per block, with
 // v_mfma_f32_16x16x32_bf16 (scores) and v_mfma_f32_16x16x16_bf16 (values):
 //   S^T = K Q^T      A = the block's 16 key rows, loaded from the pages as 16-byte pieces that are
 //                    used as they are: lane (key c, group kg) holds entries 32 kk + 8 kg .. + 7 of its
@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
     bf16_t* __restrict__ out, float* __restrict__ part, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ cache, long block_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ qsl, const int* __restrict__ seq_lens, int koff, int H, int dk, int rank, float scale,
-    const float* __restrict__ sink, int nsplit) {
+    const float* __restrict__ sink, int nsplit, int window) {
   extern __shared__ __attribute__((aligned(16))) bf16_t vt_lds[];  // [NW waves][16 VTM entries][kVtPitch] (+ [NW][KKM][64] x 16 B)
   const int s = blockIdx.z;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
@@ -68,9 +68,12 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
   const int pq = min(base + tok, last);
   const int p_first = min(base + (tile * 16) / H, last);
   const int p_last = min(base + min(tile * 16 + 15, nrows - 1) / H, last);
-  const int nblk = (p_last >> 4) + 1;
-  const int b0 = static_cast<int>(static_cast<long>(nblk) * sp / nsplit);
-  const int b1 = static_cast<int>(static_cast<long>(nblk) * (sp + 1) / nsplit);
+  // window > 0: a row at position p sees p - window + 1 .. p; the tile's walk starts at the block of
+  // its first row's oldest visible key
+  const int wb = window > 0 ? max(p_first - window + 1, 0) >> 4 : 0;
+  const int nblk = (p_last >> 4) + 1 - wb;
+  const int b0 = wb + static_cast<int>(static_cast<long>(nblk) * sp / nsplit);
+  const int b1 = wb + static_cast<int>(static_cast<long>(nblk) * (sp + 1) / nsplit);
   const int KK = EXACT ? KKM : (dk + 31) >> 5, VT = EXACT ? VTM : rank >> 4;
   const int* bt = block_tables + static_cast<long>(s) * bt_stride;
   uint4 qf[QLDS ? 1 : KKM];
@@ -138,7 +141,7 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
     const f4_t acc = (ac[0] + ac[1]) + (ac[2] + ac[3]);
     if (kb + 1 < b1) load_block(kb + 1);  // in flight while the weights are made and the values multiplied
     // a block that every row of the tile sees whole needs no mask
-    const bool whole = k0 + 15 <= p_first;
+    const bool whole = k0 + 15 <= p_first && (window <= 0 || k0 >= p_last - window + 1);
     float sv[4], mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -146,7 +149,7 @@ __global__ void __launch_bounds__(64 * NW) latent_attention_mfma_kernel(
         sv[i] = acc[i] * sl2;
       } else {
         const int j = k0 + 4 * kg + i;
-        sv[i] = (rok && j <= pq) ? acc[i] * sl2 : -INFINITY;
+        sv[i] = (rok && j <= pq && (window <= 0 || pq - j < window)) ? acc[i] * sl2 : -INFINITY;
       }
       mx = fmaxf(mx, sv[i]);
     }
@@ -224,7 +227,7 @@ __global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))
     bf16_t* __restrict__ out, float* __restrict__ part, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ cache, long block_stride, const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ qsl, const int* __restrict__ seq_lens, int koff, int H, int dk, int rank, float scale,
-    const float* __restrict__ sink, int nsplit) {
+    const float* __restrict__ sink, int nsplit, int window) {
   constexpr int KHM = KKM / 2, VHM = VTM / 2;
   static_assert(KKM % 2 == 0 && VTM % 2 == 0, "the row is split in two");
   __shared__ __attribute__((aligned(16))) bf16_t vt_s[16 * VTM * kVtPitch];
@@ -246,9 +249,12 @@ __global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int pq = min(base + tok, last);
   const int p_first = min(base + (tile * 16) / H, last);
   const int p_last = min(base + min(tile * 16 + 15, nrows - 1) / H, last);
-  const int nblk = (p_last >> 4) + 1;
-  const int b0 = static_cast<int>(static_cast<long>(nblk) * sp / nsplit);
-  const int b1 = static_cast<int>(static_cast<long>(nblk) * (sp + 1) / nsplit);
+  // window > 0: a row at position p sees p - window + 1 .. p; the tile's walk starts at the block of
+  // its first row's oldest visible key
+  const int wb = window > 0 ? max(p_first - window + 1, 0) >> 4 : 0;
+  const int nblk = (p_last >> 4) + 1 - wb;
+  const int b0 = wb + static_cast<int>(static_cast<long>(nblk) * sp / nsplit);
+  const int b1 = wb + static_cast<int>(static_cast<long>(nblk) * (sp + 1) / nsplit);
   const int KK = EXACT ? KKM : (dk + 31) >> 5, VT = EXACT ? VTM : rank >> 4;
   const int kk0 = w * KHM, vt0 = w * VHM;  // this wave's chunks and value tiles
   const int* bt = block_tables + static_cast<long>(s) * bt_stride;
@@ -315,7 +321,7 @@ __global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))
     if (kb + 1 < b1) load_block(kb + 1);  // in flight across the barrier, the weights and the value products
     __syncthreads();
     const f4_t acc = sx[buf][0][lane] + sx[buf][1][lane];  // the same sum in both waves
-    const bool whole = k0 + 15 <= p_first;
+    const bool whole = k0 + 15 <= p_first && (window <= 0 || k0 >= p_last - window + 1);
     float sv[4], mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -323,7 +329,7 @@ __global__ void __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2, 2))
         sv[i] = acc[i] * sl2;
       } else {
         const int jj = k0 + 4 * kg + i;
-        sv[i] = (rok && jj <= pq) ? acc[i] * sl2 : -INFINITY;
+        sv[i] = (rok && jj <= pq && (window <= 0 || pq - jj < window)) ? acc[i] * sl2 : -INFINITY;
       }
       mx = fmaxf(mx, sv[i]);
     }
@@ -422,7 +428,7 @@ __global__ void __launch_bounds__(128) latent_attention_combine_kernel(bf16_t* _
 bool launch_latent_attention(void* out, float* part, const void* q, long q_stride, const void* cache, long block_stride,
                              const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S, int rows,
                              int koff, int H, int dk, int rank, int bs, float scale, int max_q, const float* sink,
-                             int nsplit, bool pair, hipStream_t st) {
+                             int nsplit, bool pair, int window, hipStream_t st) {
   if (rows == 0 || S == 0) return true;
   if (bs != 16 || dk % 8 || rank % 16 || rank > dk || dk > 576 || rank > 512 || q_stride % 8 || koff % 8 ||
       block_stride % 8 || reinterpret_cast<uintptr_t>(q) % 16 || reinterpret_cast<uintptr_t>(cache) % 16 ||
@@ -433,14 +439,14 @@ bool launch_latent_attention(void* out, float* part, const void* q, long q_strid
   hipLaunchKernelGGL((latent_attention_mfma_kernel<KKM, VTM, NW, QLDS, EXACT>), dim3((tiles * nsplit + NW - 1) / NW, 1, S), \
                      dim3(64 * NW), NW * (16 * VTM * kVtPitch * sizeof(bf16_t) + (QLDS ? KKM * 64 * 16 : 0)), st,     \
                      (bf16_t*)out, part, (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, \
-                     bt_stride, qsl, seq_lens, koff, H, dk, rank, scale, sink, nsplit)
+                     bt_stride, qsl, seq_lens, koff, H, dk, rank, scale, sink, nsplit, window)
   if (dk <= 192 && rank <= 128) MIX_LA(6, 8, 4, false, false);
   else if (dk <= 320 && rank <= 256) MIX_LA(10, 16, 4, false, false);
   else if (pair) {
 #define MIX_LP(EXACT)                                                                                                  \
   hipLaunchKernelGGL((latent_attention_pair_kernel<18, 32, EXACT>), dim3(tiles * nsplit, 1, S), dim3(128), 0, st,      \
                      (bf16_t*)out, part, (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, \
-                     bt_stride, qsl, seq_lens, koff, H, dk, rank, scale, sink, nsplit)
+                     bt_stride, qsl, seq_lens, koff, H, dk, rank, scale, sink, nsplit, window)
     if (dk == 576 && rank == 512) MIX_LP(true);
     else MIX_LP(false);
 #undef MIX_LP

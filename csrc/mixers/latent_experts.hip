@@ -3,14 +3,14 @@
 // are fp32, with one rounding where a result is stored.
 //
 //   latent_prep     per token: RMS norm of the query latent; RMS norm of the key/value latent and the
-//                   half-split rotary turn of the shared key part, both written into the token's page row
+//                   rotary turn (half-split or neighbouring pairs) of the shared key part, both written into the token's page row
 //   rope_half_into  per token and head: the rotated part of the query into its columns of the folded query
-//   route_topk      sigmoid scores, the k largest per token (a wave per token)
+//   route_topk      sigmoid or softmax scores, the k largest per token (a wave per token)
 //   capped_glu      g = min(gate, L), u = clamp(up, -L, L), g * sigmoid(alpha g) * (u + 1)
 //   expert_align    counting sort of the (token, slot) pairs by expert: offsets and each pair's sorted row
 //   gather_scaled   sorted rows = routing weight * the token's input
 //   spread_scaled   [E, T, W] rows = routing weight * input for chosen experts, zero for the others
-//   expert_combine  out[t] = sum of the token's k rows (+ a shared expert's row)
+//   expert_combine  out[t] = sum of the token's k rows, each optionally times its routing weight (+ a shared expert's row)
 #include "mix_common.h"
 
 namespace mxs {
@@ -26,7 +26,7 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(
     T* __restrict__ cq, const T* __restrict__ dq, long dq_stride, const T* __restrict__ dkv, long dkv_stride,
     const int64_t* __restrict__ positions, const int64_t* __restrict__ slots, T* __restrict__ cache, long block_stride,
     int koff, int qr, int rank, int nf, int bs, const float* __restrict__ freqs, const T* __restrict__ qn,
-    const T* __restrict__ kvn, float eps) {
+    const T* __restrict__ kvn, float eps, int split) {
   __shared__ float scratch[16];
   const long t = blockIdx.x;
   const T* a = dq + t * dq_stride;
@@ -46,16 +46,18 @@ __global__ void __launch_bounds__(256) latent_prep_kernel(
   for (int i = threadIdx.x; i < nf; i += blockDim.x) {
     float sn, cs;
     sincosf(pos * freqs[i], &sn, &cs);
-    const float u = ldf(b + rank + i), v = ldf(b + rank + nf + i);
-    stf(row + rank + i, u * cs - v * sn);
-    stf(row + rank + nf + i, v * cs + u * sn);
+    // the pair's two columns: (i, i + nf) or neighbours (2i, 2i + 1)
+    const int cu = split ? i : 2 * i, cv = split ? nf + i : 2 * i + 1;
+    const float u = ldf(b + rank + cu), v = ldf(b + rank + cv);
+    stf(row + rank + cu, u * cs - v * sn);
+    stf(row + rank + cv, v * cs + u * sn);
   }
 }
 
 template <typename T>
 __global__ void __launch_bounds__(256) rope_half_into_kernel(
     T* __restrict__ out, long out_stride, const T* __restrict__ x, long x_stride, const int64_t* __restrict__ positions,
-    int heads, int x_dim, int x_col, int out_dim, int out_col, const float* __restrict__ freqs, int nf) {
+    int heads, int x_dim, int x_col, int out_dim, int out_col, const float* __restrict__ freqs, int nf, int split) {
   const long t = blockIdx.x;
   const float pos = static_cast<float>(positions[t]);
   for (int idx = threadIdx.x; idx < heads * nf; idx += blockDim.x) {
@@ -64,21 +66,32 @@ __global__ void __launch_bounds__(256) rope_half_into_kernel(
     sincosf(pos * freqs[i], &sn, &cs);
     const T* xp = x + t * x_stride + h * x_dim + x_col;
     T* op = out + t * out_stride + h * out_dim + out_col;
-    const float u = ldf(xp + i), v = ldf(xp + nf + i);
-    stf(op + i, u * cs - v * sn);
-    stf(op + nf + i, v * cs + u * sn);
+    const int cu = split ? i : 2 * i, cv = split ? nf + i : 2 * i + 1;
+    const float u = ldf(xp + cu), v = ldf(xp + cv);
+    stf(op + cu, u * cs - v * sn);
+    stf(op + cv, v * cs + u * sn);
   }
 }
 
-// A wave per token.  Scores are sigmoid(logit); the k largest are found by k passes of a wave-wide
-// arg-max over the lanes' experts (ties: the lower index), so E and k are free.
+// A wave per token.  Scores are sigmoid(logit), or the softmax over all E logits (maximum and sum by
+// the wave first); the k largest are found by k passes of a wave-wide arg-max over the lanes' experts
+// (ties: the lower index), so E and k are free.
 __global__ void __launch_bounds__(256) route_topk_kernel(float* __restrict__ w, int* __restrict__ ids,
                                                          const float* __restrict__ logits, int T, int E, int k,
-                                                         int renorm) {
+                                                         int renorm, int softmax) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (t >= T) return;  // wave-uniform
   const float* z = logits + static_cast<long>(t) * E;
+  float zmax = 0.f, zinv = 1.f;
+  if (softmax) {
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    zmax = wave_max(mx);
+    float sm = 0.f;
+    for (int e = lane; e < E; e += 64) sm += expf(z[e] - zmax);
+    zinv = 1.f / wave_sum(sm);
+  }
   float total = 0.f;
   int last_id = -1;
   float last_s = INFINITY;
@@ -87,7 +100,7 @@ __global__ void __launch_bounds__(256) route_topk_kernel(float* __restrict__ w, 
     float best = -INFINITY;
     int bi = 0x7fffffff;
     for (int e = lane; e < E; e += 64) {
-      const float sc = sigmoid_f(z[e]);
+      const float sc = softmax ? expf(z[e] - zmax) * zinv : sigmoid_f(z[e]);
       const bool after = sc < last_s || (sc == last_s && e > last_id);
       if (after && (sc > best || (sc == best && e < bi))) { best = sc; bi = e; }
     }
@@ -154,7 +167,7 @@ __global__ void __launch_bounds__(256) gather_scaled_kernel(T* __restrict__ xs, 
                                                             const float* __restrict__ w, const int* __restrict__ inv,
                                                             int k, int W) {
   const long p = blockIdx.x;
-  const float wt = w[p];
+  const float wt = w ? w[p] : 1.f;
   const T* src = h + (p / k) * h_stride;
   T* dst = xs + static_cast<long>(inv[p]) * W;
   for (int c = threadIdx.x; c < W; c += blockDim.x) stf(dst + c, ldf(src + c) * wt);
@@ -167,7 +180,7 @@ __global__ void __launch_bounds__(256) spread_scaled_kernel(T* __restrict__ xs, 
   const int t = blockIdx.x, e = blockIdx.y;
   float wt = 0.f;
   for (int j = 0; j < k; ++j)
-    if (ids[t * k + j] == e) wt += w[t * k + j];
+    if (ids[t * k + j] == e) wt += w ? w[t * k + j] : 1.f;
   const T* src = h + static_cast<long>(t) * h_stride;
   T* dst = xs + (static_cast<long>(e) * Tn + t) * W;
   for (int c = threadIdx.x; c < W; c += blockDim.x) stf(dst + c, wt == 0.f ? 0.f : ldf(src + c) * wt);
@@ -177,7 +190,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) expert_combine_kernel(T* __restrict__ out, const T* __restrict__ ys,
                                                              const int* __restrict__ index, int k, long row_stride,
                                                              const T* __restrict__ extra, long extra_stride, int W,
-                                                             int vec) {
+                                                             int vec, const float* __restrict__ wts) {
   constexpr int EL = El<T>::N;
   const long t = blockIdx.x;
   if (vec) {  // rows of whole, aligned 16-byte pieces: the k rows' loads of a piece are in flight together
@@ -194,8 +207,9 @@ __global__ void __launch_bounds__(256) expert_combine_kernel(T* __restrict__ out
         const long r = index ? index[t * k + j] : j * row_stride + t;
         float v[EL];
         load16(ys + r * W + c, v);
+        const float wt = wts ? wts[t * k + j] : 1.f;
 #pragma unroll
-        for (int e = 0; e < EL; ++e) s[e] += v[e];
+        for (int e = 0; e < EL; ++e) s[e] += wt * v[e];
       }
       store16(out + t * W + c, s);
     }
@@ -205,7 +219,7 @@ __global__ void __launch_bounds__(256) expert_combine_kernel(T* __restrict__ out
     float s = extra ? ldf(extra + t * extra_stride + c) : 0.f;
     for (int j = 0; j < k; ++j) {
       const long r = index ? index[t * k + j] : j * row_stride + t;
-      s += ldf(ys + r * W + c);
+      s += (wts ? wts[t * k + j] : 1.f) * ldf(ys + r * W + c);
     }
     stf(out + t * W + c, s);
   }
@@ -214,26 +228,29 @@ __global__ void __launch_bounds__(256) expert_combine_kernel(T* __restrict__ out
 void launch_latent_prep(void* cq, const void* dq, long dq_stride, const void* dkv, long dkv_stride,
                         const int64_t* positions, const int64_t* slots, void* cache, long block_stride, int rows, int koff,
                         int qr, int rank, int nf, int bs, const float* freqs, const void* qn, const void* kvn, float eps,
-                        bool bf, hipStream_t st) {
+                        bool split, bool bf, hipStream_t st) {
   if (rows == 0) return;
   MIX_DISPATCH(bf, hipLaunchKernelGGL(latent_prep_kernel<T>, dim3(rows), dim3(256), 0, st, (T*)cq, (const T*)dq, dq_stride,
                                       (const T*)dkv, dkv_stride, positions, slots, (T*)cache, block_stride, koff, qr, rank,
-                                      nf, bs, freqs, (const T*)qn, (const T*)kvn, eps));
+                                      nf, bs, freqs, (const T*)qn, (const T*)kvn, eps, split ? 1 : 0));
   MXS_CHECK_LAUNCH();
 }
 
 void launch_rope_half_into(void* out, long out_stride, const void* x, long x_stride, const int64_t* positions, int rows,
-                           int heads, int x_dim, int x_col, int out_dim, int out_col, const float* freqs, int nf, bool bf,
-                           hipStream_t st) {
+                           int heads, int x_dim, int x_col, int out_dim, int out_col, const float* freqs, int nf,
+                           bool split, bool bf, hipStream_t st) {
   if (rows == 0 || nf == 0) return;
   MIX_DISPATCH(bf, hipLaunchKernelGGL(rope_half_into_kernel<T>, dim3(rows), dim3(256), 0, st, (T*)out, out_stride,
-                                      (const T*)x, x_stride, positions, heads, x_dim, x_col, out_dim, out_col, freqs, nf));
+                                      (const T*)x, x_stride, positions, heads, x_dim, x_col, out_dim, out_col, freqs, nf,
+                                      split ? 1 : 0));
   MXS_CHECK_LAUNCH();
 }
 
-void launch_route_topk(float* w, int* ids, const float* logits, int T, int E, int k, bool renorm, hipStream_t st) {
+void launch_route_topk(float* w, int* ids, const float* logits, int T, int E, int k, bool renorm, bool softmax,
+                       hipStream_t st) {
   if (T == 0) return;
-  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 3) / 4), dim3(256), 0, st, w, ids, logits, T, E, k, renorm ? 1 : 0);
+  hipLaunchKernelGGL(route_topk_kernel, dim3((T + 3) / 4), dim3(256), 0, st, w, ids, logits, T, E, k, renorm ? 1 : 0,
+                     softmax ? 1 : 0);
   MXS_CHECK_LAUNCH();
 }
 
@@ -273,13 +290,13 @@ void launch_spread_scaled(void* xs, const void* h, long h_stride, const float* w
 }
 
 void launch_expert_combine(void* out, const void* ys, const int* index, int Tn, int k, long row_stride, const void* extra,
-                           long extra_stride, int W, bool bf, hipStream_t st) {
+                           long extra_stride, int W, const float* wts, bool bf, hipStream_t st) {
   if (Tn == 0) return;
   const int el = bf ? 8 : 4;
   const int vec = W % el == 0 && extra_stride % el == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
                   reinterpret_cast<uintptr_t>(ys) % 16 == 0 && reinterpret_cast<uintptr_t>(extra) % 16 == 0;
   MIX_DISPATCH(bf, hipLaunchKernelGGL(expert_combine_kernel<T>, dim3(Tn), dim3(256), 0, st, (T*)out, (const T*)ys, index, k,
-                                      row_stride, (const T*)extra, extra_stride, W, vec));
+                                      row_stride, (const T*)extra, extra_stride, W, vec, wts));
   MXS_CHECK_LAUNCH();
 }
 
