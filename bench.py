@@ -103,14 +103,15 @@ def parse(argv=None):
     # equal size (mxserve/tools/mixer_bench.py); without this flag nothing of the default workload changes
     ap.add_argument("--mixer-bench", action="store_true",
                     help="prefill / decode throughput of Voletar (or, with --mixer-design, of Tapasun beside Voletar, "
-                         "or of Momuvik beside a Mixtral-shaped model) and a Llama-shaped model of equal size, and "
+                         "of Momuvik beside a Mixtral-shaped model, or of Seradra beside both) and a Llama-shaped model "
+                         "of equal size, and "
                          "the design's kernels against their rooflines; prints JSON lines and exits")
-    ap.add_argument("--mixer-design", choices=["voletar", "tapasun", "momuvik"], default="voletar")
+    ap.add_argument("--mixer-design", choices=["voletar", "tapasun", "momuvik", "seradra"], default="voletar")
     ap.add_argument("--mixer-sizes", default="1024,2048", help="model widths, comma-separated")
     ap.add_argument("--mixer-prompt", type=int, default=4096)
     ap.add_argument("--mixer-batch", type=int, default=64)
     ap.add_argument("--mixer-context", type=int, default=2048)
-    ap.add_argument("--mixer-only", choices=["all", "momuvik", "mixtral", "tapasun", "voletar", "llama", "kernels"], default="all")
+    ap.add_argument("--mixer-only", choices=["all", "seradra", "momuvik", "mixtral", "tapasun", "voletar", "llama", "kernels"], default="all")
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--iters-per-step", type=int, default=int(os.environ.get("MXS_BENCH_ITERS_PER_STEP", "50")),

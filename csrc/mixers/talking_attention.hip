@@ -468,13 +468,27 @@ bool launch_talking_attention(void* out, const void* q, long q_stride, const voi
   const int dkp = (dk + 3) & ~3;
   const size_t shm = (static_cast<size_t>(H) * dkp + static_cast<size_t>(H) * H + 2 * static_cast<size_t>(H) * kTalkTile +
                       3 * static_cast<size_t>(H)) * sizeof(float);
-  if (shm > 64 * 1024 || H * dv > 256 * 32) return false;
+  if (shm > 160 * 1024 || H * dv > 256 * 32) return false;
   const int el = bf ? 8 : 4;
   const bool vec = dk % el == 0 && koff % el == 0 && block_stride % el == 0;
+  // many wide heads need more than the default dynamic LDS of a workgroup: asked for once per kernel
 #define MIX_TR(TT, NACC)                                                                                              \
-  hipLaunchKernelGGL((talking_attention_rows_kernel<TT, NACC>), dim3(rows), dim3(256), shm, st, (TT*)out, (const TT*)q, \
-                     q_stride, (const TT*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, koff, voff, H, \
-                     G, dk, dv, bs, scale, window, keep, vec, sink, talk)
+  do {                                                                                                                \
+    if (shm > 48 * 1024) {                                                                                            \
+      static bool raised = false;                                                                                     \
+      if (!raised) {                                                                                                  \
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&talking_attention_rows_kernel<TT, NACC>),              \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) {              \
+          (void)hipGetLastError();                                                                                    \
+          return false;                                                                                               \
+        }                                                                                                             \
+        raised = true;                                                                                                \
+      }                                                                                                               \
+    }                                                                                                                 \
+    hipLaunchKernelGGL((talking_attention_rows_kernel<TT, NACC>), dim3(rows), dim3(256), shm, st, (TT*)out, (const TT*)q, \
+                       q_stride, (const TT*)cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, koff, voff, H, \
+                       G, dk, dv, bs, scale, window, keep, vec, sink, talk);                                           \
+  } while (0)
 #define MIX_TR_T(TT)                                \
   do {                                              \
     if (H * dv <= 256 * 2) MIX_TR(TT, 2);           \

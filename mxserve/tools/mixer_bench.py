@@ -1,10 +1,11 @@
-"""Prefill and decode throughput of a layer-list design (Voletar, Tapasun, Momuvik) beside the models
+"""Prefill and decode throughput of a layer-list design (Voletar, Tapasun, Momuvik, Seradra) beside the models
 closest to it at equal width, depth and feed-forward size (random weights), through the same engine
 path: forced steps of the scheduler, the model runner, paged K/V and state slots, decode through the
 captured graphs.  Voletar stands beside a Llama-shaped model; Tapasun beside Voletar and that model;
-Momuvik beside a Mixtral-shaped model (softmax attention and routed experts of the same sizes).
+Momuvik beside a Mixtral-shaped model (softmax attention and routed experts of the same sizes); Seradra
+beside Momuvik and that model.
 
-  python bench.py --mixer-bench [--mixer-design voletar|tapasun|momuvik] [--mixer-sizes 1024,2048]
+  python bench.py --mixer-bench [--mixer-design voletar|tapasun|momuvik|seradra] [--mixer-sizes 1024,2048]
                   [--mixer-prompt 4096] [--mixer-batch 64]
 
 Prints one JSON line per (size, model): prefill tokens/s of one prompt in one step, decode tokens/s
@@ -79,7 +80,30 @@ def momuvik_shape(width: int, layers: int = 4) -> dict:
             "residual_mult": 1.0, "layers": [{"type": "latent_attention", "mixer": att, "mlp": mlp} for _ in range(layers)]}
 
 
+def seradra_shape(width: int, layers: int = 4, window: int = 1024) -> dict:
+    """Head-mixing attention (128-wide heads, 4 query heads per kv head, half of each head rotated with
+    ramp-blended frequencies) and windowed latent attention (the sizes of momuvik_shape) in turn; the first
+    layer's feed-forward is the ungated one of 4 width, the others eight experts of 4/3 width, two per token."""
+    heads = max(width // 128, 1)
+    ff = (4 * width // 3) // 256 * 256
+    att = {"heads": heads, "kv_heads": max(heads // 4, 1), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+           "mask": {"size": window}, "rot": {"dims": 64, "base": 500000.0,
+                                             "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}}
+    lat = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "q_rank": max(3 * width // 8, 256),
+           "scale": 192 ** -0.5, "mask": {"size": window}, "rot": {"dims": 64, "base": 10000.0}}
+    moe = {"kind": "moe", "router": {"experts": MOE_EXPERTS, "top": MOE_TOP}, "expert": {"ff": ff}}
+    kinds = [{"type": "attention", "mixer": att, "mlp": {"kind": "dense", "ff": 4 * width}},
+             {"type": "latent_attention", "mixer": lat, "mlp": moe}, {"type": "attention", "mixer": att, "mlp": moe},
+             {"type": "latent_attention", "mixer": lat, "mlp": moe}]
+    return {"architecture": "Seradra", "width": width, "vocab": 32000, "norm": {"eps": 1e-5},
+            "layers": [kinds[i % 4] for i in range(layers)]}
+
+
 def register(width: int, layers: int, design: str = "voletar") -> tuple:
+    if design == "seradra":
+        sd = mcfg.seradra_config(f"seradra-w{width}", seradra_shape(width, layers))
+        mcfg.REGISTRY[sd.name.lower()] = sd
+        return (sd.name,) + register(width, layers, "momuvik")
     if design == "momuvik":
         m = mcfg.momuvik_config(f"momuvik-w{width}", momuvik_shape(width, layers))
         mcfg.REGISTRY[m.name.lower()] = m
@@ -375,9 +399,107 @@ def momuvik_rooflines(width: int, prompt: int, batch: int, context: int) -> list
     return out
 
 
+def seradra_rooflines(width: int, prompt: int, batch: int, context: int) -> list:
+    """Seradra's own kernels alone, at the sizes of seradra_shape(width): time over roofline time, each beside
+    the like kernel of an existing model: the windowed attention with a sink (Voletar's / Tapasun's kernel)
+    for the head-mixing attention, Momuvik's unwindowed latent attention for the windowed one, the per-head
+    q/k/v preparation for the whole-row one, Momuvik's routed experts for the softmax-routed ones, the gated
+    activation and the fused residual kernel for the activation and the weighted sum over kept results."""
+    from ..models.feedforward import RoutedExperts
+    from ..models.mixers import rotary_frequencies
+    from ..ops import seqmix
+    dev = torch.device("cuda")
+    dt = torch.bfloat16
+    bs, out = 16, []
+    i32 = dict(dtype=torch.int32, device=dev)
+    rnd = lambda *sh: torch.randn(*sh, device=dev).to(dt)  # noqa: E731
+
+    def entry(name, t, flops, peak, bytes_, note):
+        roof = max(flops / peak, bytes_ / PEAK_HBM)
+        out.append({"kernel": name, "width": width, "ms": round(1e3 * t, 4), "roofline_ms": round(1e3 * roof, 4),
+                    "x_roofline": round(t / roof, 1), "counts": note})
+
+    shape = seradra_shape(width)["layers"]
+    ac, lc, mlp = shape[0]["mixer"], shape[1]["mixer"], shape[1]["mlp"]
+    H, G, dk, dv, win = ac["heads"], ac["kv_heads"], ac["dim"], ac["vdim"], ac["mask"]["size"]
+    rank, dr = lc["kv_rank"], lc["rot_dim"]
+    ldk = rank + dr
+    E, top, ff = MOE_EXPERTS, MOE_TOP, mlp["expert"]["ff"]
+    for mode, T, S, ctx in (("prefill", prompt, 1, prompt), ("decode", batch, batch, context)):
+        qsl = torch.arange(0, T + 1, T // S, **i32)
+        seq = torch.full((S,), ctx, **i32)
+        nb = -(-ctx // bs)
+        bt = torch.arange(S * nb, **i32).view(S, nb)
+        pos = torch.cat([torch.arange(ctx - T // S, ctx, device=dev) for _ in range(S)])
+        slots = torch.cat([bt[s_].long().repeat_interleave(bs)[ctx - T // S:ctx] * bs + pos[:T // S] % bs for s_ in range(S)])
+        keys = min(win, ctx) if mode == "decode" else min(win, ctx / 2)
+        # head-mixing attention beside the windowed attention with a sink at the same head layout
+        cache = rnd(S * nb, G * bs * (dk + dv))
+        q, k, v = rnd(T, H * dk), rnd(T, G * dk), rnd(T, G * dv)
+        sink = torch.zeros(H, device=dev)
+        talk = torch.eye(H, device=dev) + 0.1 * torch.randn(H, H, device=dev)
+        for name, tk, extra in (("talking_attention", talk, 2.0 * H), ("window_attention", None, 0.0)):
+            t = _time(lambda: seqmix.window_attention(q, cache, bt, qsl, seq, 0, G * bs * dk, H, G, dk, dv, bs, 0.09, win, 0,
+                                                      max_query_len=T // S, sink=sink, talk=tk), 5)
+            entry(f"{name}/{mode}" + ("" if tk is not None else " (voletar, tapasun)"), t, 2.0 * T * H * keys * (dk + dv), PEAK_BF16,
+                  2.0 * (S * min(win, ctx) * G * (dk + dv) + 2 * T * H * dk),
+                  f"{T} rows x {H} heads x ~{int(keys)} keys of {dk}+{dv}, bf16 MFMA peak" +
+                  (f" (the mix adds {int(extra)} fp32 multiply-adds per score, not priced)" if extra else ""))
+        fr = rotary_frequencies(64, 500000.0, ac["rot"]["scaling"]).to(dev)
+        ones = lambda n: torch.ones(n, device=dev).to(dt)  # noqa: E731
+        t = _time(lambda: seqmix.rope_qkv_cache(q, k, v, pos, slots, cache, 0, G * bs * dk, H, G, dk, dv, bs, fr, ones(H * dk),
+                                                ones(G * dk), 1e-5, bias_q=ones(H * dk), bias_k=ones(G * dk), bias_v=ones(G * dv),
+                                                norm_whole=True, split_pairs=True, mag=1.2), 5)
+        pbytes = 2.0 * T * (2 * H * dk + 2 * G * (dk + dv))
+        entry(f"qkv_prep_cache/{mode}", t, 0.0, PEAK_F32, pbytes, f"{T} rows: q read and written, k and v read and written to the pages")
+        fr2 = rotary_frequencies(64, 500000.0, None).to(dev)
+        t = _time(lambda: seqmix.rope_qkv_cache(q, k, v, pos, slots, cache, 0, G * bs * dk, H, G, dk, dv, bs, fr2, ones(dk), ones(dk),
+                                                1e-5, None), 5)
+        entry(f"rope_qkv_cache/{mode} (tapasun)", t, 0.0, PEAK_F32, pbytes, f"{T} rows: q read and written, k and v read and written to the pages")
+        # latent attention inside the window beside the unwindowed one over the whole context
+        lcache = rnd(S * nb, bs * ldk)
+        lq = rnd(T, H * ldk)
+        for name, w_, kk in (("latent_attention(window)", win, keys), ("latent_attention", 0, ctx if mode == "decode" else ctx / 2)):
+            t = _time(lambda: seqmix.latent_attention(lq, lcache, bt, qsl, seq, 0, H, ldk, rank, bs, 0.07, T // S, ctx,
+                                                      sink=None if w_ else sink, window=w_), 5)
+            entry(f"{name}/{mode}" + ("" if w_ else " (momuvik)"), t, 2.0 * T * H * kk * (ldk + rank), PEAK_BF16,
+                  2.0 * (S * (min(win, ctx) if w_ else ctx) * ldk + T * H * (ldk + rank)),
+                  f"{T} rows x {H} heads x ~{int(kk)} keys of {ldk}+{rank}, bf16 MFMA peak")
+        # routed experts: softmax scores on the outputs of plain SiLU units beside sigmoid scores on the inputs of capped ones
+        h = rnd(T, width)
+        w = {"f.router": rnd(E, width), "f._gu": rnd(E, 2 * ff, width) * width ** -0.5, "f._down": rnd(E, width, ff) * ff ** -0.5}
+        act = min(E, T * top)
+        for name, f in (("routed_experts", RoutedExperts("f.", width, E, top, ff, None, score="softmax", weigh="output")),
+                        ("routed_experts (momuvik)", RoutedExperts("f.", width, E, top, ff, 7.0))):
+            t = _time(lambda: f.forward(h, w), 5)
+            nm = name.split(" ")
+            entry(f"{nm[0]}/{mode}" + (" " + nm[1] if len(nm) > 1 else ""), t, 6.0 * T * top * width * ff, PEAK_BF16,
+                  2.0 * (3 * act * width * ff + 2 * T * width),
+                  f"{T} rows x {top} of {E} experts of {ff}, bf16 MFMA peak; {act} experts' weights read once")
+        # the ungated activation beside the gated one; the weighted sum over five kept results beside one
+        # pass of the fused residual kernel
+        z = rnd(T, 4 * width)
+        ab = torch.tensor([0.7, 1.2], device=dev)
+        t = _time(lambda: seqmix.xielu(z, ab), 5)
+        entry(f"xielu/{mode}", t, 0.0, PEAK_F32, 4.0 * T * 4 * width, f"{T} rows x {4 * width}: in and out")
+        t = _time(lambda: seqmix.silu_mul(z), 5)
+        entry(f"silu_mul/{mode} (tapasun)", t, 0.0, PEAK_F32, 3.0 * T * 4 * width, f"{T} rows x {2 * width}: gate and up in, product out")
+        hist = torch.randn(6, T, width, device=dev)
+        cf = torch.randn(5, device=dev)
+        t = _time(lambda: seqmix.depth_mix(hist, 5, cf, cast_dtype=dt), 5)
+        entry(f"depth_mix/{mode}", t, 0.0, PEAK_F32, T * width * (5 * 4.0 + 4.0 + 2.0), f"{T} rows x {width}: five fp32 slabs in, one out, one bf16 copy")
+        x = torch.randn(T, width, device=dev)
+        a = rnd(T, width)
+        t = _time(lambda: seqmix.resid_update(x, a, 1e-5, wa=ones(width), wa_offset=1.0, cast_dtype=dt), 5)
+        entry(f"resid_update/{mode}", t, 0.0, PEAK_F32, T * width * (4.0 + 2.0 + 4.0 + 2.0), f"{T} rows x {width}: stream in and out, branch in, bf16 copy out")
+        t = _time(lambda: seqmix.resid_update(x, a, 1e-5, norm_w=ones(width), out_dtype=dt, w_offset=1.0), 5)
+        entry(f"resid_update/{mode} (momuvik)", t, 0.0, PEAK_F32, T * width * (4.0 + 2.0 + 4.0 + 2.0), f"{T} rows x {width}: stream in and out, branch in, normed bf16 out")
+    return out
+
+
 def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4, only: str = "all",
          design: str = "voletar") -> int:
-    """only: all | momuvik | mixtral | tapasun | voletar | llama | kernels (e.g. one model alone under a profiler)."""
+    """only: all | seradra | momuvik | mixtral | tapasun | voletar | llama | kernels (e.g. one model alone under a profiler)."""
     from .. import ops
     ops.ext()
     for width in sizes:
@@ -386,7 +508,9 @@ def main(sizes: list, prompt: int, batch: int, context: int, layers: int = 4, on
             if only in ("all", name.split("-")[0]):
                 print(json.dumps(run_model(name, prompt, batch, context)), flush=True)
         if only in ("all", "kernels"):
-            if design == "momuvik":
+            if design == "seradra":
+                rows = seradra_rooflines(width, prompt, batch, context)
+            elif design == "momuvik":
                 rows = momuvik_rooflines(width, prompt, batch, context)
             else:
                 rows = (tapasun_rooflines(width, prompt, batch, context) if design == "tapasun" else []) + \
