@@ -18,8 +18,8 @@ void launch_qkv_prep_cache(void*, long, const void*, long, const void*, long, co
                            int, int, int, int, int, int, int, int, const float*, int, float, bool, const void*, const void*,
                            const void*, const void*, const void*, float, int, bool, hipStream_t);
 bool launch_talking_attention(void*, const void*, long, const void*, long, const int*, int, const int*, const int*, int,
-                              int, int, int, int, int, int, int, int, float, int, int, int, const float*, const float*, bool,
-                              hipStream_t);
+                              int, int, int, int, int, int, int, int, float, int, int, int, const float*, const float*, float*,
+                              int, bool, hipStream_t);
 void launch_cast_into(void*, long, const float*, int, int, bool, hipStream_t);
 void launch_relu_sq(void*, const void*, long, bool, hipStream_t);
 void launch_softcap(float*, const void*, long, int, int, float, bool, hipStream_t);
@@ -56,7 +56,7 @@ void launch_capped_glu(void*, const void*, long, int, int, float, float, bool, h
 bool launch_expert_align(int*, int*, const int*, int, int, hipStream_t);
 void launch_gather_scaled(void*, const void*, long, const float*, const int*, int, int, int, bool, hipStream_t);
 void launch_spread_scaled(void*, const void*, long, const float*, const int*, int, int, int, int, bool, hipStream_t);
-void launch_expert_combine(void*, const void*, const int*, int, int, long, const void*, long, int, const float*, bool,
+void launch_expert_combine(void*, const void*, const int*, int, int, long, const void*, long, int, const float*, bool, bool,
                            hipStream_t);
 }  // namespace mxs
 
@@ -578,7 +578,8 @@ void spread_scaled(at::Tensor xs, at::Tensor h, OptT w, at::Tensor ids) {
                             stream());
 }
 
-void expert_combine(at::Tensor out, at::Tensor ys, OptT index, int64_t k, OptT extra, int64_t row_stride, OptT weights) {
+void expert_combine(at::Tensor out, at::Tensor ys, OptT index, int64_t k, OptT extra, int64_t row_stride, OptT weights,
+                    bool by_expert) {
   const bool bf = is_bf(ys);
   TORCH_CHECK(ys.is_cuda() && ys.is_contiguous() && ys.dim() == 2 && out.is_cuda() && out.is_contiguous() &&
               out.dim() == 2 && out.size(1) == ys.size(1) && is_bf(out) == bf, "ys [R, W], out [T, W]");
@@ -587,6 +588,8 @@ void expert_combine(at::Tensor out, at::Tensor ys, OptT index, int64_t k, OptT e
   if (index.has_value()) {
     ip = i32(*index, T * k, "index");  // entries are rows of ys: expert_align's places (< T*k), or expert * T + t (< R)
     TORCH_CHECK(T * k <= R, "index reaches past ys");
+    // by_expert: entries are experts (route_topk's ids, < R / row_stride) of an [E, row_stride, W] stack
+    TORCH_CHECK(!by_expert || (row_stride >= T && R % row_stride == 0), "by_expert: ys is [E, row_stride, W]");
   } else {
     TORCH_CHECK(k >= 1 && row_stride >= T && (k - 1) * row_stride + T <= R, "the k slabs reach past ys");
   }
@@ -597,7 +600,8 @@ void expert_combine(at::Tensor out, at::Tensor ys, OptT index, int64_t k, OptT e
     wp = f32(*weights, "weights");
   }
   mxs::launch_expert_combine(out.data_ptr(), ys.data_ptr(), ip, static_cast<int>(T), static_cast<int>(k), row_stride, ep,
-                             extra.has_value() ? extra->stride(0) : 0, static_cast<int>(W), wp, bf, stream());
+                             extra.has_value() ? extra->stride(0) : 0, static_cast<int>(W), wp, by_expert && index.has_value(), bf,
+                             stream());
 }
 
 void embed_normed(at::Tensor out, OptT h, at::Tensor ids, at::Tensor table, at::Tensor w, double eps, double w_offset) {
@@ -672,7 +676,7 @@ void qkv_prep_cache(at::Tensor q, OptT k, OptT v, at::Tensor positions, at::Tens
 void talking_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tensor block_tables, at::Tensor qsl,
                        at::Tensor seq_lens, int64_t koff, int64_t voff, int64_t H, int64_t G, int64_t dk, int64_t dv,
                        int64_t bs, double scale, int64_t window, int64_t keep, int64_t max_query_len, OptT sink,
-                       at::Tensor talk) {
+                       at::Tensor talk, int64_t nsplit, OptT part) {
   const bool bf = is_bf(q);
   const float* sinkp = nullptr;
   if (sink.has_value()) {
@@ -688,14 +692,21 @@ void talking_attention(at::Tensor out, at::Tensor q, at::Tensor cache, at::Tenso
               is_bf(out) == bf, "out: [T, H*dv]");
   TORCH_CHECK(block_tables.is_cuda() && block_tables.scalar_type() == at::kInt && block_tables.dim() == 2 &&
               block_tables.size(0) >= S && block_tables.stride(1) == 1, "block_tables: int32 [S, max_blocks]");
+  float* pp = nullptr;
+  TORCH_CHECK(nsplit >= 1 && nsplit <= 64, "1 <= nsplit <= 64");
+  if (nsplit > 1) {
+    TORCH_CHECK(part.has_value() && part->numel() >= T * H * nsplit * (dv + 4), "part: fp32 [T*H, nsplit, dv + 4]");
+    pp = f32(*part, "part");
+  }
   const bool ok = mxs::launch_talking_attention(
       out.data_ptr(), mat(q, bf, T, H * dk, "q"), q.stride(0), cache.data_ptr(), cache.stride(0),
       block_tables.data_ptr<int>(), static_cast<int>(block_tables.stride(0)), i32(qsl, S + 1, "qsl"),
       i32(seq_lens, S, "seq_lens"), static_cast<int>(S), static_cast<int>(T), static_cast<int>(koff),
       static_cast<int>(voff), static_cast<int>(H), static_cast<int>(G), static_cast<int>(dk), static_cast<int>(dv),
       static_cast<int>(bs), static_cast<float>(scale), static_cast<int>(window), static_cast<int>(keep),
-      static_cast<int>(std::min<int64_t>(max_query_len, T)), sinkp, tp, bf, stream());
-  TORCH_CHECK(ok, "talking_attention: more heads or wider heads than the kernel's LDS tables hold");
+      static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(max_query_len, T))), sinkp, tp, pp, static_cast<int>(nsplit), bf,
+      stream());
+  TORCH_CHECK(ok, "talking_attention: more heads or wider heads than the kernel's LDS tables hold, or a split the sizes do not take");
 }
 
 }  // namespace

@@ -424,6 +424,16 @@ __global__ void __launch_bounds__(128) latent_attention_combine_kernel(bf16_t* _
   }
 }
 
+// The merge alone, for other attention kernels that split a row's keys over workgroups and write the same
+// (maximum in log2 units, sum, two unused, unnormalised output[width]) records: rows = (token, head) pairs.
+bool launch_attention_combine(void* out, const float* part, long rows, int nsplit, int width, hipStream_t st) {
+  if (rows == 0) return true;
+  if (nsplit < 1 || nsplit > kMaxSplit || reinterpret_cast<uintptr_t>(part) % 16) return false;
+  hipLaunchKernelGGL(latent_attention_combine_kernel, dim3(rows), dim3(128), 0, st, (bf16_t*)out, part, nsplit, width);
+  MXS_CHECK_LAUNCH();
+  return true;
+}
+
 // False: sizes the kernel does not take (the caller runs the general kernel).
 bool launch_latent_attention(void* out, float* part, const void* q, long q_stride, const void* cache, long block_stride,
                              const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S, int rows,

@@ -10,7 +10,8 @@
 //   expert_align    counting sort of the (token, slot) pairs by expert: offsets and each pair's sorted row
 //   gather_scaled   sorted rows = routing weight * the token's input
 //   spread_scaled   [E, T, W] rows = routing weight * input for chosen experts, zero for the others
-//   expert_combine  out[t] = sum of the token's k rows, each optionally times its routing weight (+ a shared expert's row)
+//   expert_combine  out[t] = sum of the token's k rows (given by place, or by expert inside an [E, T, W] stack), each
+//                   optionally times its routing weight (+ a shared expert's row)
 #include "mix_common.h"
 
 namespace mxs {
@@ -190,7 +191,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) expert_combine_kernel(T* __restrict__ out, const T* __restrict__ ys,
                                                              const int* __restrict__ index, int k, long row_stride,
                                                              const T* __restrict__ extra, long extra_stride, int W,
-                                                             int vec, const float* __restrict__ wts) {
+                                                             int vec, const float* __restrict__ wts, int by_expert) {
   constexpr int EL = El<T>::N;
   const long t = blockIdx.x;
   if (vec) {  // rows of whole, aligned 16-byte pieces: the k rows' loads of a piece are in flight together
@@ -204,7 +205,7 @@ __global__ void __launch_bounds__(256) expert_combine_kernel(T* __restrict__ out
       }
 #pragma unroll 4
       for (int j = 0; j < k; ++j) {
-        const long r = index ? index[t * k + j] : j * row_stride + t;
+        const long r = index ? (by_expert ? index[t * k + j] * row_stride + t : index[t * k + j]) : j * row_stride + t;
         float v[EL];
         load16(ys + r * W + c, v);
         const float wt = wts ? wts[t * k + j] : 1.f;
@@ -218,7 +219,7 @@ __global__ void __launch_bounds__(256) expert_combine_kernel(T* __restrict__ out
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     float s = extra ? ldf(extra + t * extra_stride + c) : 0.f;
     for (int j = 0; j < k; ++j) {
-      const long r = index ? index[t * k + j] : j * row_stride + t;
+      const long r = index ? (by_expert ? index[t * k + j] * row_stride + t : index[t * k + j]) : j * row_stride + t;
       s += (wts ? wts[t * k + j] : 1.f) * ldf(ys + r * W + c);
     }
     stf(out + t * W + c, s);
@@ -290,13 +291,13 @@ void launch_spread_scaled(void* xs, const void* h, long h_stride, const float* w
 }
 
 void launch_expert_combine(void* out, const void* ys, const int* index, int Tn, int k, long row_stride, const void* extra,
-                           long extra_stride, int W, const float* wts, bool bf, hipStream_t st) {
+                           long extra_stride, int W, const float* wts, bool by_expert, bool bf, hipStream_t st) {
   if (Tn == 0) return;
   const int el = bf ? 8 : 4;
   const int vec = W % el == 0 && extra_stride % el == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0 &&
                   reinterpret_cast<uintptr_t>(ys) % 16 == 0 && reinterpret_cast<uintptr_t>(extra) % 16 == 0;
   MIX_DISPATCH(bf, hipLaunchKernelGGL(expert_combine_kernel<T>, dim3(Tn), dim3(256), 0, st, (T*)out, (const T*)ys, index, k,
-                                      row_stride, (const T*)extra, extra_stride, W, vec, wts));
+                                      row_stride, (const T*)extra, extra_stride, W, vec, wts, by_expert ? 1 : 0));
   MXS_CHECK_LAUNCH();
 }
 

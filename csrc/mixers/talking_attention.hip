@@ -227,6 +227,11 @@ __global__ void __launch_bounds__(256) talking_attention_rows_kernel(
 //   c. O_h^T += V_g^T P_h^T with every weight as two bf16 halves; the block's value rows go through
 //      the wave's LDS area to become the key-contiguous A operand
 //   d. barrier (the raw tiles are rewritten by the next block)
+// With nsplit > 1 (steps of few rows, e.g. single decoded tokens) the visible blocks are divided over
+// nsplit workgroups; each writes (maximum, sum, unnormalised output) per row and head, and the merge
+// kernel of the latent attention combines them.
+bool launch_attention_combine(void* out, const float* part, long rows, int nsplit, int width, hipStream_t st);
+
 typedef short s4_t __attribute__((ext_vector_type(4)));
 typedef float f4_t __attribute__((ext_vector_type(4)));
 
@@ -235,14 +240,14 @@ __global__ void __launch_bounds__(64 * NW) talking_attention_mfma_kernel(
     bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ cache,
     long block_stride, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, int koff, int voff, int H, int G, int dk, int dv, float scale, int window,
-    int keep, const float* __restrict__ sink, const float* __restrict__ talk) {
+    int keep, const float* __restrict__ sink, const float* __restrict__ talk, float* __restrict__ part, int nsplit) {
   extern __shared__ __attribute__((aligned(16))) float tlds[];
   // [H][256] raw tiles (lane-major: element (lane, i) at lane * 4 + i), then [H][H] talk, then the waves' value areas
   float* raw = tlds;
   float* tk = raw + H * 256;
   const int DVP = dv + 8;
   bf16_t* vw = reinterpret_cast<bf16_t*>(tk + ((H * H + 3) & ~3)) + (threadIdx.x >> 6) * (16 * DVP);
-  const int s = blockIdx.y;
+  const int s = blockIdx.y, sp = blockIdx.z;
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
   const int row0 = qsl[s], qlen = qsl[s + 1] - row0;
   const int qt0 = blockIdx.x * 16;
@@ -266,8 +271,8 @@ __global__ void __launch_bounds__(64 * NW) talking_attention_mfma_kernel(
 #pragma unroll
     for (int ks = 0; ks < KSM; ++ks)
       qf[j][ks] = (ks < KS && qok && hok) ? *reinterpret_cast<const s4_t*>(qp + 16 * ks) : s4_t{0, 0, 0, 0};
-    m[j] = (sink && hok) ? sink[hd] * 1.4426950408889634f : -INFINITY;
-    l[j] = (sink && hok && kg == 0) ? 1.f : 0.f;
+    m[j] = (sink && hok && sp == 0) ? sink[hd] * 1.4426950408889634f : -INFINITY;  // the sink counts once: in the first stretch
+    l[j] = (sink && hok && sp == 0 && kg == 0) ? 1.f : 0.f;
 #pragma unroll
     for (int vt = 0; vt < VTM; ++vt) o[j][vt] = f4_t{0.f, 0.f, 0.f, 0.f};
   }
@@ -277,8 +282,10 @@ __global__ void __launch_bounds__(64 * NW) talking_attention_mfma_kernel(
   const int kA = window > 0 ? min((keep + 15) >> 4, wb) : 0;
   const float sl2 = scale * 1.4426950408889634f;
   const int nit = kA + (lastb - wb + 1);
+  const int it0 = static_cast<int>(static_cast<long>(nit) * sp / nsplit);
+  const int it1 = static_cast<int>(static_cast<long>(nit) * (sp + 1) / nsplit);
   __syncthreads();
-  for (int it = 0; it < nit; ++it) {
+  for (int it = it0; it < it1; ++it) {
     const int kb = it < kA ? it : wb + (it - kA);
     const bf16_t* blk = cache + static_cast<long>(bt[kb]) * block_stride;
     const int k0 = kb * 16;
@@ -389,6 +396,14 @@ __global__ void __launch_bounds__(64 * NW) talking_attention_mfma_kernel(
     lj += __shfl_xor(lj, 16, 64);
     lj += __shfl_xor(lj, 32, 64);
     if (hd >= H || !qok) continue;
+    if (nsplit > 1) {
+      float* pp = part + ((static_cast<long>(row0 + qt0 + c) * H + hd) * nsplit + sp) * (dv + 4);
+      if (kg == 0) { pp[0] = m[j]; pp[1] = lj; }
+#pragma unroll
+      for (int vt = 0; vt < VTM; ++vt)
+        if (vt < VT) *reinterpret_cast<f4_t*>(pp + 4 + 16 * vt + 4 * kg) = o[j][vt];
+      continue;
+    }
     const float inv = 1.f / lj;
     bf16_t* op = out + static_cast<long>(row0 + qt0 + c) * (H * dv) + hd * dv + 4 * kg;
 #pragma unroll
@@ -421,7 +436,7 @@ template <int KSM, int VTM, int HPW, int NW>
 static bool launch_talking_mfma(void* out, const void* q, long q_stride, const void* cache, long block_stride,
                                 const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S, int koff,
                                 int voff, int H, int G, int dk, int dv, float scale, int window, int keep, int max_q,
-                                const float* sink, const float* talk, hipStream_t st) {
+                                const float* sink, const float* talk, float* part, int nsplit, hipStream_t st) {
   const size_t shm = (static_cast<size_t>(H) * 256 + ((H * H + 3) & ~3)) * sizeof(float) +
                      static_cast<size_t>(NW) * 16 * (dv + 8) * sizeof(bf16_t);
   if (shm > 160 * 1024) return false;
@@ -436,9 +451,9 @@ static bool launch_talking_mfma(void* out, const void* q, long q_stride, const v
       raised = true;
     }
   }
-  hipLaunchKernelGGL((talking_attention_mfma_kernel<KSM, VTM, HPW, NW>), dim3((max_q + 15) / 16, S), dim3(64 * NW), shm, st,
-                     (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride,
-                     qsl, seq_lens, koff, voff, H, G, dk, dv, scale, window, keep, sink, talk);
+  hipLaunchKernelGGL((talking_attention_mfma_kernel<KSM, VTM, HPW, NW>), dim3((max_q + 15) / 16, S, nsplit), dim3(64 * NW),
+                     shm, st, (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables,
+                     bt_stride, qsl, seq_lens, koff, voff, H, G, dk, dv, scale, window, keep, sink, talk, part, nsplit);
   MXS_CHECK_LAUNCH();
   return true;
 }
@@ -446,15 +461,17 @@ static bool launch_talking_mfma(void* out, const void* q, long q_stride, const v
 bool launch_talking_attention(void* out, const void* q, long q_stride, const void* cache, long block_stride,
                               const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S, int rows,
                               int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep,
-                              int max_q, const float* sink, const float* talk, bool bf, hipStream_t st) {
+                              int max_q, const float* sink, const float* talk, float* part, int nsplit, bool bf,
+                              hipStream_t st) {
   if (rows == 0 || S == 0) return true;
-  // prompt chunks in bf16 with MFMA-shaped heads: the matrix-core form (a mixed step's single tokens ride
-  // along as 1-row tiles)
-  if (bf && max_q >= 16 && bs == 16 && dk % 16 == 0 && dv % 16 == 0 && dk <= 128 && dv <= 128 && q_stride % 4 == 0 &&
+  if (nsplit < 1 || (nsplit > 1 && (part == nullptr || reinterpret_cast<uintptr_t>(part) % 16))) return false;
+  // bf16 with MFMA-shaped heads: the matrix-core form for prompt chunks and single tokens alike (a single
+  // token is a 1-row tile; steps of few rows split every row's keys over nsplit workgroups)
+  if (bf && max_q >= 1 && bs == 16 && dk % 16 == 0 && dv % 16 == 0 && dk <= 128 && dv <= 128 && q_stride % 4 == 0 &&
       reinterpret_cast<uintptr_t>(q) % 8 == 0 && koff % 8 == 0 && voff % 8 == 0 && block_stride % 8 == 0 && H <= 64) {
 #define MIX_TA(KSM, VTM, HPW, NW)                                                                                       \
   launch_talking_mfma<KSM, VTM, HPW, NW>(out, q, q_stride, cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, \
-                                         koff, voff, H, G, dk, dv, scale, window, keep, max_q, sink, talk, st)
+                                         koff, voff, H, G, dk, dv, scale, window, keep, max_q, sink, talk, part, nsplit, st)
     const bool small = dk <= 64 && dv <= 64;
     bool done = false;
     if (H <= 4) done = small ? MIX_TA(4, 4, 1, 4) : MIX_TA(8, 8, 1, 4);
@@ -463,8 +480,9 @@ bool launch_talking_attention(void* out, const void* q, long q_stride, const voi
     else if (H <= 32) done = small ? MIX_TA(4, 4, 2, 16) : MIX_TA(8, 8, 2, 16);
     else done = small ? MIX_TA(4, 4, 4, 16) : false;
 #undef MIX_TA
-    if (done) return true;
+    if (done) return nsplit == 1 || launch_attention_combine(out, part, static_cast<long>(rows) * H, nsplit, dv, st);
   }
+  // the rows form walks a row's keys in one workgroup, whatever split was asked for
   const int dkp = (dk + 3) & ~3;
   const size_t shm = (static_cast<size_t>(H) * dkp + static_cast<size_t>(H) * H + 2 * static_cast<size_t>(H) * kTalkTile +
                       3 * static_cast<size_t>(H)) * sizeof(float);

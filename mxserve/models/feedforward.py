@@ -163,8 +163,7 @@ class RoutedExperts(FeedForward):
             if w_out is None:
                 return seqmix.expert_combine(ys, None, self.E, T, extra, row_stride=T)
             # weights on the outputs: a token's k chosen slabs, row (expert, t) of the stack
-            index = (ids * T + torch.arange(T, dtype=torch.int32, device=ids.device).view(T, 1)).reshape(-1)
-            return seqmix.expert_combine(ys, index, self.top, T, extra, weights=w_out)
+            return seqmix.expert_combine(ys, ids.reshape(-1), self.top, T, extra, row_stride=T, weights=w_out, by_expert=True)
         offs, inv = seqmix.expert_align(ids, self.E)
         xs = seqmix.gather_scaled(h, w_in, inv, self.top)
         ys = torch.empty_like(xs)

@@ -618,7 +618,8 @@ class TalkingAttention(Mixer):
                               norm_whole=self.whole_norm, split_pairs=True, mag=self.mag)
         o = seqmix.window_attention(q, ctx.cache, md.block_tables, md.query_start_loc, md.seq_lens, koff, voff,
                                     self.heads, self.kv_heads, self.dk, self.dv, ctx.block_size, self.scale, self.window,
-                                    0, md.max_query_len, sink=w.get(p + "sink"), talk=w.get(p + "talk"))
+                                    0, md.max_query_len, sink=w.get(p + "sink"), talk=w.get(p + "talk"),
+                                    max_seq_len=getattr(md, "max_seq_len", 0))
         return ops.linear(o, w[p + "o"])
 
 

@@ -194,6 +194,9 @@ def gate_linear(h: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor]) 
 
 
 # ----------------------------------------------------------------------------- windowed attention
+TALK_TARGET_GROUPS = 512  # workgroups (all heads of 16 rows each) that fill the 256 CUs two deep: steps of few rows split their keys up to this
+
+
 def kv_write(cache: torch.Tensor, k: torch.Tensor, v: torch.Tensor, slot_mapping: torch.Tensor, koff: int,
              voff: int, num_kv_heads: int, dk: int, dv: int, block_size: int) -> None:
     """k [T, Hkv*dk], v [T, Hkv*dv] (row-strided views) into the paged cache; slot -1 writes nothing."""
@@ -214,7 +217,7 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
                      seq_lens: torch.Tensor, koff: int, voff: int, num_heads: int, num_kv_heads: int, dk: int,
                      dv: int, block_size: int, scale: float, window: int, keep_first: int,
                      max_query_len: int = 0, sink: Optional[torch.Tensor] = None, v_stride: int = 0,
-                     talk: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     talk: Optional[torch.Tensor] = None, max_seq_len: int = 0) -> torch.Tensor:
     """Softmax attention over the paged cache (this step's keys already written).  The query at
     position i sees key j <= i when i - j < window or j < keep_first (window <= 0: every j <= i).
     q [T, H*dk] (row-strided view) -> [T, H*dv] in q's dtype; scores and weights in fp32.
@@ -225,15 +228,26 @@ def window_attention(q: torch.Tensor, cache: torch.Tensor, block_tables: torch.T
     int); from 16 rows a bf16 step with head sizes that are multiples of 16 runs the MFMA kernel.
     talk (fp32 [H, H]): the heads' scaled scores of a (query, key) pair are mixed before the softmax,
     score_h <- sum_g talk[h, g] score_g (the mask and the sink act on the mixed scores); a workgroup then
-    serves all heads of its rows."""
+    serves all heads of its rows, and a bf16 step of few rows splits every row's keys over several
+    workgroups (max_seq_len, a host int, bounds how many are worth it) whose stretches are merged."""
     T = q.shape[0]
     if _gpu(q) and talk is not None:
         if v_stride and v_stride != dv:
             raise ValueError("mixed heads read value rows back to back")
         out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
+        nsplit, part = 1, None
+        if q.dtype == torch.bfloat16 and T and block_size == 16 and dk % 16 == 0 and dv % 16 == 0 and dk <= 128 and dv <= 128:
+            mq = max(1, min(int(max_query_len) or T, T))
+            tiles = seq_lens.numel() * (-(-mq // 16))
+            span = int(max_seq_len) or 16
+            if window > 0:
+                span = min(span, int(window) + int(keep_first) + 15)
+            nsplit = max(1, min(16, TALK_TARGET_GROUPS // max(tiles, 1), -(-span // 16) // 2))
+            if nsplit > 1:
+                part = torch.empty(T * num_heads * nsplit * (dv + 4), dtype=torch.float32, device=q.device)
         ext().talking_attention(out, q, cache, block_tables, qsl, seq_lens, int(koff), int(voff), num_heads, num_kv_heads,
                                 dk, dv, block_size, float(scale), int(window), int(keep_first), int(max_query_len), sink,
-                                talk)
+                                talk, nsplit, part)
         return out
     if _gpu(q):
         out = torch.empty(T, num_heads * dv, dtype=q.dtype, device=q.device)
@@ -839,18 +853,21 @@ def spread_scaled(h: torch.Tensor, weights: Optional[torch.Tensor], ids: torch.T
 
 
 def expert_combine(ys: torch.Tensor, index: Optional[torch.Tensor], k: int, T: int, extra: Optional[torch.Tensor] = None,
-                   row_stride: int = 0, weights: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   row_stride: int = 0, weights: Optional[torch.Tensor] = None, by_expert: bool = False) -> torch.Tensor:
     """out[t] = sum_j ys[index[t*k + j]] (+ extra[t]); index None: row j*row_stride + t (the k slabs
-    of a [k, T, W] stack).  weights (fp32 [T, k]): row j of token t enters times weights[t, j] (routing
-    weights on the experts' outputs).  Summed in fp32, rounded once."""
+    of a [k, T, W] stack); by_expert: index holds experts and the row is index[t*k + j]*row_stride + t (a
+    token's chosen slabs of an [E, T, W] stack).  weights (fp32 [T, k]): row j of token t enters times
+    weights[t, j] (routing weights on the experts' outputs).  Summed in fp32, rounded once."""
     W = ys.shape[-1]
     y2 = ys.reshape(-1, W)
     if _gpu(ys):
         out = torch.empty(T, W, dtype=ys.dtype, device=ys.device)
-        ext().expert_combine(out, y2, index, int(k), extra, int(row_stride), weights)
+        ext().expert_combine(out, y2, index, int(k), extra, int(row_stride), weights, bool(by_expert))
         return out
     if index is None:
         idx = (torch.arange(k).view(1, k) * row_stride + torch.arange(T).view(T, 1)).reshape(-1)
+    elif by_expert:
+        idx = (index.long().view(T, k) * row_stride + torch.arange(T).view(T, 1)).reshape(-1)
     else:
         idx = index.long()
     rows = y2[idx].float().view(T, k, W)

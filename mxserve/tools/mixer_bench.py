@@ -440,21 +440,20 @@ def seradra_rooflines(width: int, prompt: int, batch: int, context: int) -> list
         talk = torch.eye(H, device=dev) + 0.1 * torch.randn(H, H, device=dev)
         for name, tk, extra in (("talking_attention", talk, 2.0 * H), ("window_attention", None, 0.0)):
             t = _time(lambda: seqmix.window_attention(q, cache, bt, qsl, seq, 0, G * bs * dk, H, G, dk, dv, bs, 0.09, win, 0,
-                                                      max_query_len=T // S, sink=sink, talk=tk), 5)
+                                                      max_query_len=T // S, sink=sink, talk=tk, max_seq_len=ctx), 5)
             entry(f"{name}/{mode}" + ("" if tk is not None else " (voletar, tapasun)"), t, 2.0 * T * H * keys * (dk + dv), PEAK_BF16,
                   2.0 * (S * min(win, ctx) * G * (dk + dv) + 2 * T * H * dk),
                   f"{T} rows x {H} heads x ~{int(keys)} keys of {dk}+{dv}, bf16 MFMA peak" +
                   (f" (the mix adds {int(extra)} fp32 multiply-adds per score, not priced)" if extra else ""))
         fr = rotary_frequencies(64, 500000.0, ac["rot"]["scaling"]).to(dev)
         ones = lambda n: torch.ones(n, device=dev).to(dt)  # noqa: E731
-        t = _time(lambda: seqmix.rope_qkv_cache(q, k, v, pos, slots, cache, 0, G * bs * dk, H, G, dk, dv, bs, fr, ones(H * dk),
-                                                ones(G * dk), 1e-5, bias_q=ones(H * dk), bias_k=ones(G * dk), bias_v=ones(G * dv),
-                                                norm_whole=True, split_pairs=True, mag=1.2), 5)
+        oq, ok_, ov, od, ow = ones(H * dk), ones(G * dk), ones(G * dv), ones(dk), ones(width)
+        t = _time(lambda: seqmix.rope_qkv_cache(q, k, v, pos, slots, cache, 0, G * bs * dk, H, G, dk, dv, bs, fr, oq, ok_, 1e-5,
+                                                bias_q=oq, bias_k=ok_, bias_v=ov, norm_whole=True, split_pairs=True, mag=1.2), 5)
         pbytes = 2.0 * T * (2 * H * dk + 2 * G * (dk + dv))
         entry(f"qkv_prep_cache/{mode}", t, 0.0, PEAK_F32, pbytes, f"{T} rows: q read and written, k and v read and written to the pages")
         fr2 = rotary_frequencies(64, 500000.0, None).to(dev)
-        t = _time(lambda: seqmix.rope_qkv_cache(q, k, v, pos, slots, cache, 0, G * bs * dk, H, G, dk, dv, bs, fr2, ones(dk), ones(dk),
-                                                1e-5, None), 5)
+        t = _time(lambda: seqmix.rope_qkv_cache(q, k, v, pos, slots, cache, 0, G * bs * dk, H, G, dk, dv, bs, fr2, od, od, 1e-5, None), 5)
         entry(f"rope_qkv_cache/{mode} (tapasun)", t, 0.0, PEAK_F32, pbytes, f"{T} rows: q read and written, k and v read and written to the pages")
         # latent attention inside the window beside the unwindowed one over the whole context
         lcache = rnd(S * nb, bs * ldk)
@@ -490,9 +489,9 @@ def seradra_rooflines(width: int, prompt: int, batch: int, context: int) -> list
         entry(f"depth_mix/{mode}", t, 0.0, PEAK_F32, T * width * (5 * 4.0 + 4.0 + 2.0), f"{T} rows x {width}: five fp32 slabs in, one out, one bf16 copy")
         x = torch.randn(T, width, device=dev)
         a = rnd(T, width)
-        t = _time(lambda: seqmix.resid_update(x, a, 1e-5, wa=ones(width), wa_offset=1.0, cast_dtype=dt), 5)
+        t = _time(lambda: seqmix.resid_update(x, a, 1e-5, wa=ow, wa_offset=1.0, cast_dtype=dt), 5)
         entry(f"resid_update/{mode}", t, 0.0, PEAK_F32, T * width * (4.0 + 2.0 + 4.0 + 2.0), f"{T} rows x {width}: stream in and out, branch in, bf16 copy out")
-        t = _time(lambda: seqmix.resid_update(x, a, 1e-5, norm_w=ones(width), out_dtype=dt, w_offset=1.0), 5)
+        t = _time(lambda: seqmix.resid_update(x, a, 1e-5, norm_w=ow, out_dtype=dt, w_offset=1.0), 5)
         entry(f"resid_update/{mode} (momuvik)", t, 0.0, PEAK_F32, T * width * (4.0 + 2.0 + 4.0 + 2.0), f"{T} rows x {width}: stream in and out, branch in, normed bf16 out")
     return out
 

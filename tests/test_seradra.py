@@ -150,6 +150,8 @@ TALKING_SHAPES = [
     talking(heads=5, kv_heads=5, dim=32, vdim=16, scale=0.12, window=1000, rot_dims=6, scaling=None),
     talking(heads=20, kv_heads=4, dim=16, vdim=16, scale=0.2, window=35, rot_dims=8),
     talking(heads=8, kv_heads=8, dim=80, vdim=96, scale=0.1, window=17, rot_dims=32),
+    talking(heads=18, kv_heads=6, dim=96, vdim=80, scale=0.1, window=30, rot_dims=64),
+    talking(heads=40, kv_heads=10, dim=16, vdim=32, scale=0.25, window=50, rot_dims=4, scaling=None),
 ]
 
 
@@ -158,7 +160,7 @@ TALKING_SHAPES = [
 def test_talking_attention_mixer(dev, dtype, portions):
     """Several shapes: grouped key/value heads, one head of one rotary pair that sees itself only, a
     rotation over the whole head, a window longer than the sequence, more heads than a workgroup has
-    waves, heads wider than 64."""
+    waves (two and four heads a wave), heads wider than 64."""
     _skip(dev)
     width, T = 72, 70
     h = torch.randn(T, width, generator=torch.Generator().manual_seed(1))
