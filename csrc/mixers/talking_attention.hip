@@ -11,6 +11,8 @@
 //                    fp32, single decoded tokens
 //   talking_attention (MFMA form)   bf16 prompt chunks: a workgroup owns 16 query rows, one wave per head
 //                    (or several heads a wave); raw score tiles are exchanged through LDS
+//   talking_attention (single-token MFMA form)   bf16 steps of single tokens: a workgroup owns one row, a wave
+//                    one kv head (or several), a tile's columns are that kv head's query heads
 // Scores, the mix, maxima, sums and output accumulators are fp32.
 #include "mix_common.h"
 
@@ -307,7 +309,7 @@ __global__ void __launch_bounds__(64 * NW) talking_attention_mfma_kernel(
           for (int i = 0; i < 4; ++i)
             if (k0 + 4 * kg + i > p_last) acc[i] = 0.f;
         }
-        *reinterpret_cast<f4_t*>(raw + hd * 256 + lane * 4) = acc;
+        if (qok) *reinterpret_cast<f4_t*>(raw + hd * 256 + lane * 4) = acc;  // a 1-row tile moves a sixteenth of the tile
       }
     }
     __syncthreads();
@@ -320,11 +322,13 @@ __global__ void __launch_bounds__(64 * NW) talking_attention_mfma_kernel(
       // b. mix and softmax
       f4_t mx4 = f4_t{0.f, 0.f, 0.f, 0.f};
       const float* trow = tk + hd * H;
-      for (int g = 0; g < H; ++g) {
-        const f4_t r = *reinterpret_cast<const f4_t*>(raw + g * 256 + lane * 4);
-        const float tw = trow[g];
+      if (qok) {  // lanes of rows the tile does not have read nothing: single tokens need a sixteenth of the LDS traffic
+        for (int g = 0; g < H; ++g) {
+          const f4_t r = *reinterpret_cast<const f4_t*>(raw + g * 256 + lane * 4);
+          const float tw = trow[g];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) mx4[i] += tw * r[i];
+          for (int i = 0; i < 4; ++i) mx4[i] += tw * r[i];
+        }
       }
       float sv[4], mx = -INFINITY;
 #pragma unroll
@@ -418,6 +422,183 @@ __global__ void __launch_bounds__(64 * NW) talking_attention_mfma_kernel(
   }
 }
 
+// ---- Single-token form (bf16, same sizes): a workgroup owns ONE query row.  The 16 columns of a tile are
+// the R = H / G query heads of one kv head (R <= 16) instead of 16 rows of one head, and wave w serves the
+// kv heads w, w + NW, ...: a block's keys and values are loaded and multiplied once per kv head, not once
+// per query head, and R of the 16 columns do useful work instead of one.  The raw scores are [H][16 keys]
+// in LDS; the mix, the softmax and the split over nsplit workgroups are those of the form above.
+template <int KSM, int VTM, int GPW, int NW>
+__global__ void __launch_bounds__(64 * NW) talking_attention_token_kernel(
+    bf16_t* __restrict__ out, const bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ cache,
+    long block_stride, const int* __restrict__ block_tables, int bt_stride, const int* __restrict__ qsl,
+    const int* __restrict__ seq_lens, int S, int koff, int voff, int H, int G, int dk, int dv, float scale, int window,
+    int keep, const float* __restrict__ sink, const float* __restrict__ talk, float* __restrict__ part, int nsplit) {
+  extern __shared__ __attribute__((aligned(16))) float tlds[];
+  float* raw = tlds;            // [H][16]
+  float* tk = raw + H * 16;     // [H][H]
+  const int DVP = dv + 8;
+  bf16_t* vw = reinterpret_cast<bf16_t*>(tk + ((H * H + 3) & ~3)) + (threadIdx.x >> 6) * (16 * DVP);
+  const int t = blockIdx.x, sp = blockIdx.y;
+  const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6;
+  const int s = seq_of_row(qsl, S, t);
+  const int qlen = qsl[s + 1] - qsl[s];
+  const int pos = min(max(seq_lens[s] - qlen + (t - qsl[s]), 0), bt_stride * 16 - 1);
+  const int c = lane & 15, kg = lane >> 4;
+  const int KS = dk >> 4, VT = dv >> 4, R = H / G;
+  const bool qok = c < R;
+  const int* bt = block_tables + static_cast<long>(s) * bt_stride;
+  for (int i = threadIdx.x; i < H * H; i += blockDim.x) tk[i] = talk[i];
+  s4_t qf[GPW][KSM];
+  float m[GPW], l[GPW];
+  f4_t o[GPW][VTM];
+#pragma unroll
+  for (int j = 0; j < GPW; ++j) {
+    const int g = wid + j * NW;
+    const bool ok = qok && g < G;
+    const int hd = ok ? g * R + c : 0;
+    const bf16_t* qp = q + static_cast<long>(t) * q_stride + hd * dk + 4 * kg;
+#pragma unroll
+    for (int ks = 0; ks < KSM; ++ks)
+      qf[j][ks] = (ks < KS && ok) ? *reinterpret_cast<const s4_t*>(qp + 16 * ks) : s4_t{0, 0, 0, 0};
+    m[j] = (sink && ok && sp == 0) ? sink[hd] * 1.4426950408889634f : -INFINITY;
+    l[j] = (sink && ok && sp == 0 && kg == 0) ? 1.f : 0.f;
+#pragma unroll
+    for (int vt = 0; vt < VTM; ++vt) o[j][vt] = f4_t{0.f, 0.f, 0.f, 0.f};
+  }
+  const int lo_first = window > 0 ? max(pos - window + 1, 0) : 0;
+  const int wb = lo_first >> 4, lastb = pos >> 4;
+  const int kA = window > 0 ? min((keep + 15) >> 4, wb) : 0;
+  const float sl2 = scale * 1.4426950408889634f;
+  const int nit = kA + (lastb - wb + 1);
+  const int it0 = static_cast<int>(static_cast<long>(nit) * sp / nsplit);
+  const int it1 = static_cast<int>(static_cast<long>(nit) * (sp + 1) / nsplit);
+  __syncthreads();
+  for (int it = it0; it < it1; ++it) {
+    const int kb = it < kA ? it : wb + (it - kA);
+    const bf16_t* blk = cache + static_cast<long>(bt[kb]) * block_stride;
+    const int k0 = kb * 16;
+#pragma unroll
+    for (int j = 0; j < GPW; ++j) {
+      const int g = wid + j * NW;
+      if (g < G) {
+        f4_t acc = f4_t{0.f, 0.f, 0.f, 0.f};
+        const bf16_t* kp = blk + koff + (static_cast<long>(g) * 16 + c) * dk + 4 * kg;
+#pragma unroll
+        for (int ks = 0; ks < KSM; ++ks)
+          if (ks < KS)
+            acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const s4_t*>(kp + 16 * ks), qf[j][ks], acc, 0, 0, 0);
+        if (k0 + 15 > pos) {  // stale rows behind the sequence's end: zeros, before they can meet the mix
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (k0 + 4 * kg + i > pos) acc[i] = 0.f;
+        }
+        if (qok) *reinterpret_cast<f4_t*>(raw + (g * R + c) * 16 + 4 * kg) = acc;
+      }
+    }
+    __syncthreads();
+    const bool whole = k0 + 15 <= pos && (window <= 0 || k0 >= pos - window + 1 || k0 + 15 < keep);
+    const bool vall = k0 + 15 <= pos;
+#pragma unroll
+    for (int j = 0; j < GPW; ++j) {
+      const int g = wid + j * NW;
+      if (g >= G) continue;  // wave-uniform
+      f4_t mx4 = f4_t{0.f, 0.f, 0.f, 0.f};
+      if (qok) {
+        const float* trow = tk + (g * R + c) * H;
+        for (int g2 = 0; g2 < H; ++g2) {
+          const f4_t r = *reinterpret_cast<const f4_t*>(raw + g2 * 16 + 4 * kg);
+          const float tw = trow[g2];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mx4[i] += tw * r[i];
+        }
+      }
+      float sv[4], mx = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int jk = k0 + 4 * kg + i;
+        const bool vis = qok && (whole || (jk <= pos && (window <= 0 || pos - jk < window || jk < keep)));
+        sv[i] = vis ? mx4[i] * sl2 : -INFINITY;
+        mx = fmaxf(mx, sv[i]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[j], mx);
+      if (__builtin_amdgcn_ballot_w64(m_new > m[j]) != 0) {
+        const float corr = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m[j] - m_new);
+        l[j] *= corr;
+#pragma unroll
+        for (int vt = 0; vt < VTM; ++vt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[j][vt][i] *= corr;
+        m[j] = m_new;
+      }
+      s4_t ph, pl;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pr = sv[i] != -INFINITY ? __builtin_amdgcn_exp2f(sv[i] - m[j]) : 0.f;
+        l[j] += pr;
+        const uint32_t u = __float_as_uint(pr), uh = u & 0xFFFF0000u;
+        uint32_t ul = __float_as_uint(pr - __uint_as_float(uh));
+        ul += 0x7FFFu + ((ul >> 16) & 1u);
+        ph[i] = static_cast<short>(uh >> 16);
+        pl[i] = static_cast<short>(ul >> 16);
+      }
+      const bf16_t* vblk = blk + voff + static_cast<long>(g) * 16 * dv;
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int r = 0; r < (VTM + 1) / 2; ++r) {
+        const int idx = lane + 64 * r;
+        if (idx < 2 * dv) {
+          const int e0 = idx * 8, vr = e0 / dv, vc = e0 - vr * dv;
+          *reinterpret_cast<uint4*>(vw + vr * DVP + vc) = *reinterpret_cast<const uint4*>(vblk + e0);
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+      const bf16_t* vp = vw + 4 * kg * DVP + c;
+#pragma unroll
+      for (int vt = 0; vt < VTM; ++vt) {
+        if (vt < VT) {
+          s4_t a;
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            a[i] = (vall || k0 + 4 * kg + i <= pos) ? static_cast<short>(vp[i * DVP + 16 * vt]) : short(0);
+          const f4_t tt = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, ph, o[j][vt], 0, 0, 0);
+          o[j][vt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, pl, tt, 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int j = 0; j < GPW; ++j) {
+    const int g = wid + j * NW;
+    float lj = l[j];
+    lj += __shfl_xor(lj, 16, 64);
+    lj += __shfl_xor(lj, 32, 64);
+    if (g >= G || !qok) continue;
+    const int hd = g * R + c;
+    if (nsplit > 1) {
+      float* pp = part + ((static_cast<long>(t) * H + hd) * nsplit + sp) * (dv + 4);
+      if (kg == 0) { pp[0] = m[j]; pp[1] = lj; }
+#pragma unroll
+      for (int vt = 0; vt < VTM; ++vt)
+        if (vt < VT) *reinterpret_cast<f4_t*>(pp + 4 + 16 * vt + 4 * kg) = o[j][vt];
+      continue;
+    }
+    const float inv = 1.f / lj;
+    bf16_t* op = out + static_cast<long>(t) * (H * dv) + hd * dv + 4 * kg;
+#pragma unroll
+    for (int vt = 0; vt < VTM; ++vt) {
+      if (vt < VT) {
+        uint2 w;
+        w.x = pack2(o[j][vt][0] * inv, o[j][vt][1] * inv);
+        w.y = pack2(o[j][vt][2] * inv, o[j][vt][3] * inv);
+        *reinterpret_cast<uint2*>(op + 16 * vt) = w;
+      }
+    }
+  }
+}
+
 void launch_qkv_prep_cache(void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
                            const int64_t* positions, const int64_t* slots, void* cache, long block_stride, int rows,
                            int koff, int voff, int H, int G, int dk, int dv, int bs, const float* freqs, int nf, float mag,
@@ -458,6 +639,32 @@ static bool launch_talking_mfma(void* out, const void* q, long q_stride, const v
   return true;
 }
 
+template <int KSM, int VTM, int GPW, int NW>
+static bool launch_talking_token(void* out, const void* q, long q_stride, const void* cache, long block_stride,
+                                 const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S, int rows,
+                                 int koff, int voff, int H, int G, int dk, int dv, float scale, int window, int keep,
+                                 const float* sink, const float* talk, float* part, int nsplit, hipStream_t st) {
+  const size_t shm = (static_cast<size_t>(H) * 16 + ((H * H + 3) & ~3)) * sizeof(float) +
+                     static_cast<size_t>(NW) * 16 * (dv + 8) * sizeof(bf16_t);
+  if (shm > 160 * 1024) return false;
+  if (shm > 48 * 1024) {
+    static bool raised = false;
+    if (!raised) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(&talking_attention_token_kernel<KSM, VTM, GPW, NW>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) {
+        (void)hipGetLastError();
+        return false;
+      }
+      raised = true;
+    }
+  }
+  hipLaunchKernelGGL((talking_attention_token_kernel<KSM, VTM, GPW, NW>), dim3(rows, nsplit), dim3(64 * NW), shm, st,
+                     (bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)cache, block_stride, block_tables, bt_stride,
+                     qsl, seq_lens, S, koff, voff, H, G, dk, dv, scale, window, keep, sink, talk, part, nsplit);
+  MXS_CHECK_LAUNCH();
+  return true;
+}
+
 bool launch_talking_attention(void* out, const void* q, long q_stride, const void* cache, long block_stride,
                               const int* block_tables, int bt_stride, const int* qsl, const int* seq_lens, int S, int rows,
                               int koff, int voff, int H, int G, int dk, int dv, int bs, float scale, int window, int keep,
@@ -469,11 +676,27 @@ bool launch_talking_attention(void* out, const void* q, long q_stride, const voi
   // token is a 1-row tile; steps of few rows split every row's keys over nsplit workgroups)
   if (bf && max_q >= 1 && bs == 16 && dk % 16 == 0 && dv % 16 == 0 && dk <= 128 && dv <= 128 && q_stride % 4 == 0 &&
       reinterpret_cast<uintptr_t>(q) % 8 == 0 && koff % 8 == 0 && voff % 8 == 0 && block_stride % 8 == 0 && H <= 64) {
+    const bool small = dk <= 64 && dv <= 64;
+    bool done = false;
+    if (max_q == 1 && H / G <= 16) {  // single tokens only: a tile's columns are the query heads of a kv head
+#define MIX_TT(KSM, VTM, GPW, NW)                                                                                       \
+  launch_talking_token<KSM, VTM, GPW, NW>(out, q, q_stride, cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, \
+                                          rows, koff, voff, H, G, dk, dv, scale, window, keep, sink, talk, part, nsplit, st)
+#define MIX_TT_N(GPW, NW) (small ? MIX_TT(4, 4, GPW, NW) : MIX_TT(8, 8, GPW, NW))
+      if (G <= 1) done = MIX_TT_N(1, 1);
+      else if (G <= 2) done = MIX_TT_N(1, 2);
+      else if (G <= 4) done = MIX_TT_N(1, 4);
+      else if (G <= 8) done = MIX_TT_N(1, 8);
+      else if (G <= 16) done = MIX_TT_N(1, 16);
+      else if (G <= 32) done = MIX_TT_N(2, 16);
+      else done = small ? MIX_TT(4, 4, 4, 16) : false;
+#undef MIX_TT_N
+#undef MIX_TT
+      if (done) return nsplit == 1 || launch_attention_combine(out, part, static_cast<long>(rows) * H, nsplit, dv, st);
+    }
 #define MIX_TA(KSM, VTM, HPW, NW)                                                                                       \
   launch_talking_mfma<KSM, VTM, HPW, NW>(out, q, q_stride, cache, block_stride, block_tables, bt_stride, qsl, seq_lens, S, \
                                          koff, voff, H, G, dk, dv, scale, window, keep, max_q, sink, talk, part, nsplit, st)
-    const bool small = dk <= 64 && dv <= 64;
-    bool done = false;
     if (H <= 4) done = small ? MIX_TA(4, 4, 1, 4) : MIX_TA(8, 8, 1, 4);
     else if (H <= 8) done = small ? MIX_TA(4, 4, 1, 8) : MIX_TA(8, 8, 1, 8);
     else if (H <= 16) done = small ? MIX_TA(4, 4, 1, 16) : MIX_TA(8, 8, 1, 16);
