@@ -10,7 +10,7 @@
 namespace mxs {
 void launch_resid_update(float*, const void*, long, const void*, const void*, long, const void*, const void*, int,
                          const void*, void*, int, int, float, float, float, float, bool, hipStream_t);
-void launch_embed_normed(float*, void*, const int64_t*, const void*, const void*, int, int, long, float, float, bool,
+void launch_embed_normed(float*, float*, void*, const int64_t*, const void*, const void*, int, int, long, float, float, bool,
                          hipStream_t);
 bool launch_depth_mix(float*, long, int, const float*, void*, int, int, bool, hipStream_t);
 void launch_xielu(void*, const void*, long, const float*, bool, hipStream_t);
@@ -604,8 +604,14 @@ void expert_combine(at::Tensor out, at::Tensor ys, OptT index, int64_t k, OptT e
                              stream());
 }
 
-void embed_normed(at::Tensor out, OptT h, at::Tensor ids, at::Tensor table, at::Tensor w, double eps, double w_offset) {
+void embed_normed(at::Tensor out, OptT copy, OptT h, at::Tensor ids, at::Tensor table, at::Tensor w, double eps,
+                  double w_offset) {
   float* op = f32(out, "out");
+  float* cp = nullptr;
+  if (copy.has_value()) {
+    cp = f32(*copy, "copy");
+    TORCH_CHECK(copy->sizes() == out.sizes(), "copy: fp32 [T, W] like out");
+  }
   TORCH_CHECK(table.is_cuda() && table.dim() == 2 && table.is_contiguous(), "table: contiguous [vocab, W]");
   const bool bf = is_bf(table);
   const int64_t T = ids.numel(), W = table.size(1);
@@ -616,7 +622,7 @@ void embed_normed(at::Tensor out, OptT h, at::Tensor ids, at::Tensor table, at::
                 "h: contiguous [T, W] of the table's dtype");
     hp = h->data_ptr();
   }
-  mxs::launch_embed_normed(op, hp, i64c(ids, T, "ids"), table.data_ptr(), vec(OptT(w), bf, W, "w"), static_cast<int>(T),
+  mxs::launch_embed_normed(op, cp, hp, i64c(ids, T, "ids"), table.data_ptr(), vec(OptT(w), bf, W, "w"), static_cast<int>(T),
                            static_cast<int>(W), table.size(0), static_cast<float>(eps), static_cast<float>(w_offset), bf,
                            stream());
 }

@@ -12,12 +12,13 @@ namespace mxs {
     else { using T = float; __VA_ARGS__; }         \
   } while (0)
 
-// out[t] = RMSNorm(table[ids[t]]) * (w_offset + w); h (optional) = the same rounded to T.
+// out[t] = RMSNorm(table[ids[t]]) * (w_offset + w); h (optional) = the same rounded to T; copy (optional) = a
+// second fp32 copy (the slab the first layer updates in place).
 template <typename T>
-__global__ void __launch_bounds__(256) embed_normed_kernel(float* __restrict__ out, T* __restrict__ h,
-                                                           const int64_t* __restrict__ ids, const T* __restrict__ table,
-                                                           const T* __restrict__ w, int W, long vocab, float eps,
-                                                           float w_offset) {
+__global__ void __launch_bounds__(256) embed_normed_kernel(float* __restrict__ out, float* __restrict__ copy,
+                                                           T* __restrict__ h, const int64_t* __restrict__ ids,
+                                                           const T* __restrict__ table, const T* __restrict__ w, int W,
+                                                           long vocab, float eps, float w_offset) {
   __shared__ float scratch[16];
   const long t = blockIdx.x;
   long id = ids[t];
@@ -29,6 +30,7 @@ __global__ void __launch_bounds__(256) embed_normed_kernel(float* __restrict__ o
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     const float v = ldf(row + c) * inv * (w_offset + ldf(w + c));
     out[t * W + c] = v;
+    if (copy) copy[t * W + c] = v;
     if (h) stf(h + t * W + c, v);
   }
 }
@@ -81,10 +83,10 @@ __global__ void __launch_bounds__(256) xielu_kernel(T* __restrict__ out, const T
   }
 }
 
-void launch_embed_normed(float* out, void* h, const int64_t* ids, const void* table, const void* w, int rows, int W,
+void launch_embed_normed(float* out, float* copy, void* h, const int64_t* ids, const void* table, const void* w, int rows, int W,
                          long vocab, float eps, float w_offset, bool bf, hipStream_t st) {
   if (rows == 0) return;
-  MIX_DISPATCH(bf, hipLaunchKernelGGL(embed_normed_kernel<T>, dim3(rows), dim3(256), 0, st, out, (T*)h, ids,
+  MIX_DISPATCH(bf, hipLaunchKernelGGL(embed_normed_kernel<T>, dim3(rows), dim3(256), 0, st, out, copy, (T*)h, ids,
                                       (const T*)table, (const T*)w, W, vocab, eps, w_offset));
   MXS_CHECK_LAUNCH();
 }

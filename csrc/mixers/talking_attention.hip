@@ -29,8 +29,8 @@ namespace mxs {
 template <typename T>
 __device__ __forceinline__ void prep_row(const T* __restrict__ src, T* __restrict__ dst, int heads, int dk,
                                          const T* __restrict__ bias, const T* __restrict__ nw, int norm_mode,
-                                         float eps, const float* __restrict__ freqs, int nf, int split, float mag,
-                                         float pos, float* __restrict__ rh, float* __restrict__ scratch, bool write,
+                                         float eps, const float* __restrict__ cs_t, const float* __restrict__ sn_t,
+                                         int nf, int split, float* __restrict__ rh, float* __restrict__ scratch, bool write,
                                          long head_stride) {
   // src: the projection's row [heads * dk]; dst: element (hd, c) goes to dst[hd * head_stride + c]
   const int lane = threadIdx.x & 63, wid = threadIdx.x >> 6, nw_ = blockDim.x >> 6;
@@ -66,10 +66,7 @@ __device__ __forceinline__ void prep_row(const T* __restrict__ src, T* __restric
   for (int idx = threadIdx.x; idx < heads * nf; idx += blockDim.x) {
     const int hd = idx / nf, p = idx - hd * nf;
     const int cu = split ? p : 2 * p, cv = split ? p + nf : 2 * p + 1;
-    float sn, cs;
-    sincosf(pos * freqs[p], &sn, &cs);
-    sn *= mag;
-    cs *= mag;
+    const float sn = sn_t[p], cs = cs_t[p];  // the pair's turn, made once per token for all heads
     const float u = val(hd, cu), v = val(hd, cv);
     stf(dst + hd * head_stride + cu, u * cs - v * sn);
     stf(dst + hd * head_stride + cv, v * cs + u * sn);
@@ -88,20 +85,32 @@ __global__ void __launch_bounds__(256) qkv_prep_cache_kernel(
     int koff, int voff, int H, int G, int dk, int dv, int bs, const float* __restrict__ freqs, int nf, float mag,
     int split, const T* __restrict__ bq, const T* __restrict__ bk, const T* __restrict__ bv, const T* __restrict__ qn,
     const T* __restrict__ kn, float eps, int norm_mode) {
-  extern __shared__ float rh[];  // [max(H, G)] per-head inverse rms
+  extern __shared__ float rh[];  // [max(H, G)] per-head inverse rms, then cos [nf] and sin [nf] of the token's turns
   __shared__ float scratch[16];
   const long t = blockIdx.x;
   const float pos = static_cast<float>(positions[t]);
-  T* qr = q + t * q_stride;
-  prep_row<T>(qr, qr, H, dk, bq, qn, norm_mode, eps, freqs, nf, split, mag, pos, rh, scratch, true, dk);
-  if (k == nullptr) return;
+  float* cs_t = rh + max(H, G);
+  float* sn_t = cs_t + nf;
+  for (int p = threadIdx.x; p < nf; p += blockDim.x) {
+    float sn, cs;
+    sincosf(pos * freqs[p], &sn, &cs);
+    cs_t[p] = cs * mag;
+    sn_t[p] = sn * mag;
+  }
+  __syncthreads();
+  // blockIdx.y == 0: the queries; 1: keys and values (two workgroups a token, so that single-token steps,
+  // which are a chain of dependent passes, run the two chains side by side)
+  if (blockIdx.y == 0) {
+    T* qr = q + t * q_stride;
+    prep_row<T>(qr, qr, H, dk, bq, qn, norm_mode, eps, cs_t, sn_t, nf, split, rh, scratch, true, dk);
+    return;
+  }
   const int64_t slot = slots[t];
   const bool wr = slot >= 0;  // a padding row writes nothing (block-uniform)
   T* base = cache + (wr ? slot / bs : 0) * block_stride;
   const int off = wr ? static_cast<int>(slot % bs) : 0;
-  __syncthreads();  // rh is reused
-  prep_row<T>(k + t * k_stride, base + koff + static_cast<long>(off) * dk, G, dk, bk, kn, norm_mode, eps, freqs, nf, split,
-              mag, pos, rh, scratch, wr, static_cast<long>(bs) * dk);
+  prep_row<T>(k + t * k_stride, base + koff + static_cast<long>(off) * dk, G, dk, bk, kn, norm_mode, eps, cs_t, sn_t, nf,
+              split, rh, scratch, wr, static_cast<long>(bs) * dk);
   if (!wr) return;
   const T* vr = v + t * v_stride;
   for (int i = threadIdx.x; i < G * dv; i += blockDim.x) {
@@ -605,8 +614,8 @@ void launch_qkv_prep_cache(void* q, long q_stride, const void* k, long k_stride,
                            bool split, const void* bq, const void* bk, const void* bv, const void* qn, const void* kn,
                            float eps, int norm_mode, bool bf, hipStream_t st) {
   if (rows == 0) return;
-  const size_t shm = static_cast<size_t>(std::max(H, G)) * sizeof(float);
-  MIX_DISPATCH(bf, hipLaunchKernelGGL(qkv_prep_cache_kernel<T>, dim3(rows), dim3(256), shm, st, (T*)q, q_stride, (const T*)k,
+  const size_t shm = static_cast<size_t>(std::max(H, G) + 2 * nf) * sizeof(float);
+  MIX_DISPATCH(bf, hipLaunchKernelGGL(qkv_prep_cache_kernel<T>, dim3(rows, k ? 2 : 1), dim3(256), shm, st, (T*)q, q_stride, (const T*)k,
                                       k_stride, (const T*)v, v_stride, positions, slots, (T*)cache, block_stride, koff, voff,
                                       H, G, dk, dv, bs, freqs, nf, mag, split ? 1 : 0, (const T*)bq, (const T*)bk,
                                       (const T*)bv, (const T*)qn, (const T*)kn, eps, norm_mode));

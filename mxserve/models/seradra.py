@@ -148,8 +148,7 @@ class SeradraLM(HybridLM):
         # slab 0: the embedding output; slab n + 1: what run n produced; a run starts from the weighted sum
         # that the run before it left in its slab
         hist = torch.empty(len(runs) + 2, T, self.width, dtype=torch.float32, device=w["embed"].device)
-        h = seqmix.embed_normed(input_ids, w["embed"], w["embed.norm"], eps, 1.0, hist[0], cast_dtype=dt)
-        hist[1].copy_(hist[0])
+        h = seqmix.embed_normed(input_ids, w["embed"], w["embed.norm"], eps, 1.0, hist[0], cast_dtype=dt, copy=hist[1])
         tap = self.layer_tap
         for n, run in enumerate(runs):
             i = run.layer

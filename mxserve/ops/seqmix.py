@@ -103,14 +103,17 @@ def resid_update(x: torch.Tensor, a: Optional[torch.Tensor], eps: float, *, wa: 
 
 
 def embed_normed(ids: torch.Tensor, table: torch.Tensor, w: torch.Tensor, eps: float, w_offset: float,
-                 out: torch.Tensor, cast_dtype: Optional[torch.dtype] = None):
+                 out: torch.Tensor, cast_dtype: Optional[torch.dtype] = None, copy: Optional[torch.Tensor] = None):
     """out (fp32 [T, W], may be one slab of a larger buffer) = RMSNorm(table[ids]) * (w_offset + w): an
-    embedding that is normed before it becomes the stream.  Returns out in cast_dtype when asked."""
+    embedding that is normed before it becomes the stream; `copy` receives the same (a second slab that a
+    layer then updates in place).  Returns out in cast_dtype when asked."""
     if _gpu(table):
         h = torch.empty(out.shape, dtype=cast_dtype, device=out.device) if cast_dtype is not None else None
-        ext().embed_normed(out, h, ids, table, w, float(eps), float(w_offset))
+        ext().embed_normed(out, copy, h, ids, table, w, float(eps), float(w_offset))
         return h
     out.copy_(_rms(F.embedding(ids, table).float(), eps) * (w.float() + w_offset))
+    if copy is not None:
+        copy.copy_(out)
     return None if cast_dtype is None else out.to(cast_dtype, copy=True)
 
 

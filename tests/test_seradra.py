@@ -511,12 +511,12 @@ def test_stream_of_kept_results(dev):
         ids = torch.tensor([3, 0, 10, 3, 7])
         hist = torch.full((4, 5, W), float("nan"))
         hs = hist.to(dev)
-        h0 = seqmix.embed_normed(ids.to(dev), table.to(dev), wn.to(dev), 1e-3, 1.0, hs[0], cast_dtype=torch.float32)
+        h0 = seqmix.embed_normed(ids.to(dev), table.to(dev), wn.to(dev), 1e-3, 1.0, hs[0], cast_dtype=torch.float32, copy=hs[1])
         e = table[ids].double()
         x0 = e / torch.sqrt((e ** 2).mean(-1, keepdim=True) + 1e-3) * (1.0 + wn.double())
         assert torch.allclose(hs[0].cpu().double(), x0, atol=1e-5) and torch.allclose(h0.cpu().double(), x0, atol=1e-5)
+        assert torch.equal(hs[1], hs[0])
         a = 3.0 * torch.randn(5, W, generator=g)
-        hs[1].copy_(hs[0])
         hn = seqmix.resid_update(hs[1], a.to(dev), 1e-3, wa=wn.to(dev), wa_offset=1.0, cast_dtype=torch.float32)
         x1 = x0 + a.double() / torch.sqrt((a.double() ** 2).mean(-1, keepdim=True) + 1e-3) * (1.0 + wn.double())
         assert torch.allclose(hs[1].cpu().double(), x1, atol=1e-5) and torch.allclose(hn.cpu().double(), x1, atol=1e-5)
