@@ -145,7 +145,7 @@ PORTIONS = [[1000], [1], [2], [5, 1, 9, 2, 30]]
 TALKING_SHAPES = [
     talking(),
     talking(heads=1, kv_heads=1, dim=2, vdim=3, scale=0.7, window=1, rot_dims=2, base=50.0, scaling=None),
-    talking(heads=6, kv_heads=2, dim=20, vdim=12, scale=0.15, window=16, rot_dims=20, base=250000.0,
+    talking(heads=6, kv_heads=2, dim=20, vdim=12, scale=0.15, window=16, rot_dims=20, base=200000.0,
             scaling={"factor": 8.0, "original": 32, "fast": 4.0, "slow": 0.5}),
     talking(heads=5, kv_heads=5, dim=32, vdim=16, scale=0.12, window=1000, rot_dims=6, scaling=None),
     talking(heads=20, kv_heads=4, dim=16, vdim=16, scale=0.2, window=35, rot_dims=8),
@@ -179,7 +179,7 @@ def test_talking_attention_mixer(dev, dtype, portions):
 LATENT_SHAPES = [
     latent(),
     latent(heads=1, dim=8, rot_dim=2, vdim=8, kv_rank=8, q_rank=8, scale=0.5, window=1, base=50.0),
-    latent(heads=6, dim=16, rot_dim=32, vdim=24, kv_rank=136, q_rank=16, scale=0.1, window=16, base=250000.0),
+    latent(heads=6, dim=16, rot_dim=32, vdim=24, kv_rank=136, q_rank=16, scale=0.1, window=16, base=200000.0),
     latent(heads=2, dim=72, rot_dim=8, vdim=8, kv_rank=24, q_rank=100, scale=0.12, window=500),
     latent(heads=4, dim=32, rot_dim=16, vdim=32, kv_rank=64, q_rank=48, scale=0.15, window=37),
     latent(heads=3, dim=10, rot_dim=6, vdim=7, kv_rank=13, q_rank=9, scale=0.3, window=20),
