@@ -153,6 +153,7 @@ TALKING_SHAPES = [
     talking(heads=18, kv_heads=6, dim=96, vdim=80, scale=0.1, window=30, rot_dims=64),
     talking(heads=40, kv_heads=10, dim=16, vdim=32, scale=0.25, window=50, rot_dims=4, scaling=None),
     talking(heads=34, kv_heads=2, dim=16, vdim=16, scale=0.25, window=28, rot_dims=16, scaling=None),
+    talking(heads=2, kv_heads=1, dim=144, vdim=136, scale=0.08, window=45, rot_dims=100),
 ]
 
 
@@ -161,7 +162,8 @@ TALKING_SHAPES = [
 def test_talking_attention_mixer(dev, dtype, portions):
     """Several shapes: grouped key/value heads, one head of one rotary pair that sees itself only, a
     rotation over the whole head, a window longer than the sequence, more heads than a workgroup has
-    waves (two and four heads a wave), heads wider than 64, more query heads per kv head than a tile has columns."""
+    waves (two and four heads a wave), heads wider than 64, more query heads per kv head than a tile has columns, heads wider than the
+    matrix-core forms take."""
     _skip(dev)
     width, T = 72, 70
     h = torch.randn(T, width, generator=torch.Generator().manual_seed(1))
